@@ -1,0 +1,197 @@
+"""GPU parity of the elementwise, reduction, softmax and matmul entry points.
+
+Cases and tolerances follow the reference's own unit tests
+(tests/test_gpu_op.py:5-182): exact for set/broadcast/relu masks, rtol 1e-5 for
+sums, softmax and matmul at the reference's shapes.
+"""
+import numpy as np
+import pytest
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu(a, rt):
+    from tinyflow_amd import ndarray
+    return ndarray.array(np.asarray(a, dtype=np.float32), rt.ctx)
+
+
+def _empty(shape, rt):
+    from tinyflow_amd import ndarray
+    return ndarray.empty(shape, rt.ctx)
+
+
+def test_array_roundtrip_and_set(rt):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(0)
+    for shape in [(1,), (3,), (5, 7), (2000, 2500), (2, 3, 5, 7), (1025,)]:
+        x = rng.uniform(-1, 1, shape).astype(np.float32)
+        a = _gpu(x, rt)
+        assert a.shape == shape
+        np.testing.assert_array_equal(a.asnumpy(), x)
+        gpu_op.array_set(a, 3.25, rt.stream)
+        np.testing.assert_array_equal(a.asnumpy(), np.full(shape, 3.25, np.float32))
+
+
+@pytest.mark.parametrize("shape", [(1,), (7,), (500, 200), (2000, 2500), (3, 5, 7, 11), (64, 256, 56, 56)])
+def test_elementwise(rt, shape):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(1)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    y = rng.uniform(-1, 1, shape).astype(np.float32)
+    x.flat[::7] = 0.0  # exact zeros for the relu mask
+    a, b, c = _gpu(x, rt), _gpu(y, rt), _empty(shape, rt)
+    gpu_op.matrix_elementwise_add(a, b, c, rt.stream)
+    np.testing.assert_array_equal(c.asnumpy(), O.add(x, y))
+    gpu_op.matrix_elementwise_multiply(a, b, c, rt.stream)
+    np.testing.assert_array_equal(c.asnumpy(), O.multiply(x, y))
+    gpu_op.matrix_elementwise_add_by_const(a, 0.37, c, rt.stream)
+    np.testing.assert_array_equal(c.asnumpy(), O.add_by_const(x, 0.37))
+    gpu_op.matrix_elementwise_multiply_by_const(a, -1.5, c, rt.stream)
+    np.testing.assert_array_equal(c.asnumpy(), O.multiply_by_const(x, -1.5))
+    gpu_op.relu(a, c)
+    np.testing.assert_array_equal(c.asnumpy(), O.relu(x))
+    gpu_op.relu_gradient(a, b, c)
+    np.testing.assert_array_equal(c.asnumpy(), O.relu_gradient(x, y))
+    # mask is x > 0: nothing passes at exact zeros
+    assert np.all(c.asnumpy().flat[::7] == 0)
+    # SGD in place; a*b+c may or may not be fused, so allow one rounding
+    w = _gpu(x, rt)
+    gpu_op.sgd_update(w, b, 0.01, rt.stream)
+    np.testing.assert_allclose(w.asnumpy(), O.sgd_update(x, y, 0.01), rtol=1e-6, atol=1e-7)
+
+
+def test_broadcast(rt):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(2)
+    b = rng.uniform(-1, 1, (100,)).astype(np.float32)
+    out = _empty((128, 100), rt)
+    gpu_op.broadcast_to(_gpu(b, rt), out, "NHWC", rt.stream)
+    np.testing.assert_array_equal(out.asnumpy(), O.broadcast_to_trailing(b, (128, 100)))
+    for shape in [(4, 6, 28, 28), (3, 5, 7, 9), (2, 16, 10, 10)]:
+        b = rng.uniform(-1, 1, (shape[1],)).astype(np.float32)
+        out = _empty(shape, rt)
+        gpu_op.broadcast_to(_gpu(b, rt), out, "NCHW", rt.stream)
+        np.testing.assert_array_equal(out.asnumpy(), O.broadcast_to_channel(b, shape))
+
+
+@pytest.mark.parametrize("shape", [(500, 200, 100), (128, 256), (1000, 10), (7,), (64, 1000), (100000, 3)])
+def test_reduce_sum_axis_zero(rt, shape):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(3)
+    x = rng.uniform(0, 20, shape).astype(np.float32)
+    out_shape = shape[1:] if len(shape) > 1 else (1,)
+    out = _empty(out_shape, rt)
+    gpu_op.reduce_sum_axis_zero(_gpu(x, rt), out)
+    ref = np.sum(x.astype(np.float64), axis=0).reshape(out_shape)
+    np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape,fmt", [((128, 256), "NHWC"), ((128, 10), "NHWC"), ((64, 6, 28, 28), "NCHW"),
+                                      ((32, 64, 56, 56), "NCHW"), ((5, 3, 7, 9), "NCHW"), ((2, 16, 10, 10), "NCHW")])
+def test_bias_gradient_reduce_sum(rt, shape, fmt):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(4)
+    dy = rng.normal(0, 1, shape).astype(np.float32)
+    C = shape[1]
+    in_s, out_s = gpu_op.reduce_sum_get_real_shape(shape, (C,), fmt)
+    lst = gpu_op.reduce_sum_get_cudnnlist(in_s, out_s, fmt, rt.cudnn)
+    out = _empty((C,), rt)
+    assert gpu_op.reduce_sum_new(_gpu(dy, rt), out, lst, rt.cudnn, rt.stream) == 0
+    ref = O.bias_gradient(dy.astype(np.float64), fmt)
+    np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-4, atol=1e-4)
+    # legacy entry points compute the same sums
+    out2 = _empty((C,), rt)
+    gpu_op.broadcast_to_backward(_gpu(dy, rt), out2, fmt)
+    np.testing.assert_allclose(out2.asnumpy(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape", [(400, 1000), (128, 10), (64, 1000), (1, 3), (5000, 17)])
+def test_softmax_and_cross_entropy(rt, shape):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(5)
+    y = rng.uniform(-5, 5, shape).astype(np.float32)
+    labels = np.zeros(shape, np.float32)
+    labels[np.arange(shape[0]), rng.randint(0, shape[1], shape[0])] = 1
+    out = _empty(shape, rt)
+    gpu_op.softmax(_gpu(y, rt), out, rt.stream)
+    np.testing.assert_allclose(out.asnumpy(), O.softmax(y), rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(out.asnumpy().sum(axis=1), 1.0, rtol=1e-5)
+    loss = _empty((1,), rt)
+    gpu_op.softmax_cross_entropy(_gpu(y, rt), _gpu(labels, rt), loss, rt.stream)
+    np.testing.assert_allclose(loss.asnumpy(), O.softmax_cross_entropy(y.astype(np.float64), labels), rtol=1e-5)
+
+
+MM_CASES = [
+    # the reference's own cases (tests/test_gpu_op.py:103-131)
+    ((500, 700), False, (700, 1000), False),
+    ((1000, 700), False, (500, 700), True),   # NT
+    ((700, 500), True, (1000, 700), True),    # TT
+    # MLP config shapes: forward, dA = dZ W^T, dW = A^T dZ
+    ((128, 784), False, (784, 256), False),
+    ((128, 256), False, (784, 256), True),
+    ((128, 784), True, (128, 256), False),
+    ((128, 100), False, (100, 10), False),
+    # ragged edges and tiny sizes
+    ((3, 2), False, (2, 3), False),
+    ((1, 1), False, (1, 1), False),
+    ((65, 17), False, (17, 129), False),
+    ((33, 130), True, (33, 70), False),
+    # skinny with a long reduction (split-k path)
+    ((32, 4096), False, (4096, 1000), False),
+    ((64, 2048), False, (2048, 1000), False),
+    ((64, 2048), True, (64, 1000), False),
+]
+
+
+@pytest.mark.parametrize("sa,ta,sb,tb", MM_CASES)
+def test_matmul(rt, sa, ta, sb, tb):
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(6)
+    a = rng.uniform(-1, 1, sa).astype(np.float32)
+    b = rng.uniform(-1, 1, sb).astype(np.float32)
+    ref = O.matmul(a.astype(np.float64), ta, b.astype(np.float64), tb)
+    c = _empty(ref.shape, rt)
+    gpu_op.matrix_multiply(_gpu(a, rt), ta, _gpu(b, rt), tb, c, rt.cublas, rt.stream)
+    np.testing.assert_allclose(c.asnumpy(), ref, rtol=1e-5, atol=1e-4)
+
+
+def test_matmul_reference_integer_case(rt):
+    """3x2 . 2x3 integer matrices and their gradients with a ones upstream
+    (reference tests/autodiff_test.py:188-208)."""
+    from tinyflow_amd import gpu_op
+    x2 = np.array([[1, 2], [3, 4], [5, 6]], np.float32)
+    x3 = np.array([[7, 8, 9], [10, 11, 12]], np.float32)
+    y = _empty((3, 3), rt)
+    gpu_op.matrix_multiply(_gpu(x2, rt), False, _gpu(x3, rt), False, y, rt.cublas, rt.stream)
+    np.testing.assert_array_equal(y.asnumpy(), np.matmul(x2, x3))
+    ones = np.ones((3, 3), np.float32)
+    d2, d3 = _empty((3, 2), rt), _empty((2, 3), rt)
+    gpu_op.matrix_multiply(_gpu(ones, rt), False, _gpu(x3, rt), True, d2, rt.cublas, rt.stream)
+    gpu_op.matrix_multiply(_gpu(x2, rt), True, _gpu(ones, rt), False, d3, rt.cublas, rt.stream)
+    np.testing.assert_array_equal(d2.asnumpy(), np.matmul(ones, x3.T))
+    np.testing.assert_array_equal(d3.asnumpy(), np.matmul(x2.T, ones))
+
+
+def test_alloc_oom_convention(rt):
+    """An allocation the device cannot serve reports the byte count (as a
+    32-bit int) and returns no array (reference ndarray.py:251-259)."""
+    from tinyflow_amd import ndarray
+    ret = ndarray.empty((1 << 20, 1 << 20), rt.ctx)  # 4 TiB
+    assert isinstance(ret, int)
+
+
+def test_copy_with_stream_and_d2d(rt):
+    from tinyflow_amd import ndarray
+    rng = np.random.RandomState(7)
+    x = rng.normal(0, 1, (257, 129)).astype(np.float32)
+    a = _gpu(x, rt)
+    b = _empty(x.shape, rt)
+    a.copyto(b, rt.stream)  # device to device on the compute stream
+    np.testing.assert_array_equal(b.asnumpy(), x)
+    host = ndarray.empty(x.shape, ndarray.cpu(0))  # pinned
+    b.copyto(host, rt.stream)
+    np.testing.assert_array_equal(host.asnumpy(), x)
+    c = host.copyto(rt.ctx, rt.stream)
+    np.testing.assert_array_equal(c.asnumpy(), x)

@@ -1,0 +1,355 @@
+// Bandwidth-bound elementwise kernels: array set, add / multiply (tensor and
+// constant), ReLU and its gradient, broadcasts, cross-entropy terms, SGD and Adam.
+//
+// All of them stream their operands once: each lane moves 16-byte vectors,
+// four independent vectors are in flight per lane and the grid is sized to the
+// CU count with a grid-stride loop, so a launch is bounded by HBM bandwidth
+// (8 or 12 bytes per element) rather than by the number of workgroups.
+//
+// Reference kernels replaced: src/gpu_op.cu:39-52 (set, broadcast),
+// :108-123 (channel broadcast), :193-235 (add/mul/relu), :4461-4533 (Adam),
+// :4538-4597 (cross), :4600-4625 (SGD); one thread per element, 1024-thread
+// blocks capped at 4096 blocks there.
+#include "internal.h"
+
+using namespace tf;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+struct OpSet { float v; __device__ float operator()(float, float) const { return v; } };
+struct OpAdd { __device__ float operator()(float a, float b) const { return a + b; } };
+struct OpMul { __device__ float operator()(float a, float b) const { return a * b; } };
+struct OpAddC { float v; __device__ float operator()(float a, float) const { return a + v; } };
+struct OpMulC { float v; __device__ float operator()(float a, float) const { return a * v; } };
+struct OpRelu { __device__ float operator()(float a, float) const { return a < 0.f ? 0.f : a; } };
+// gradient mask is x > 0 (reference kernel gpu_op.cu:230-235 and its test
+// tests/test_gpu_op.py:145-155); a = x, b = upstream gradient
+struct OpReluGrad { __device__ float operator()(float a, float b) const { return a > 0.f ? b : 0.f; } };
+// a = parameter, b = gradient
+struct OpSgd { float lr; __device__ float operator()(float a, float b) const { return a - lr * b; } };
+// a = x (probabilities), b = y (labels)
+struct OpCross { float s; __device__ float operator()(float a, float b) const { return logf(a) * b * (-1.f) * s; } };
+
+template <class F>
+__device__ inline float4 apply4(const F &f, const float4 &a, const float4 &b) {
+  return make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w));
+}
+
+// out[i] = f(a[i], b[i]) over n4 float4 vectors plus a scalar tail.
+// out may alias a (in-place SGD), so no restrict qualifiers.
+template <class F, bool HAS_A, bool HAS_B>
+__global__ __launch_bounds__(kThreads) void ew_kernel(F f, float *out, const float *a, const float *b,
+                                                     int64_t n4, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const float4 *a4 = reinterpret_cast<const float4 *>(a);
+  const float4 *b4 = reinterpret_cast<const float4 *>(b);
+  float4 *o4 = reinterpret_cast<float4 *>(out);
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (; i + (kUnroll - 1) * stride < n4; i += kUnroll * stride) {
+    float4 va[kUnroll], vb[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      va[u] = HAS_A ? a4[i + u * stride] : zero;
+      vb[u] = HAS_B ? b4[i + u * stride] : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) o4[i + u * stride] = apply4(f, va[u], vb[u]);
+  }
+  for (; i < n4; i += stride) {
+    const float4 va = HAS_A ? a4[i] : zero;
+    const float4 vb = HAS_B ? b4[i] : zero;
+    o4[i] = apply4(f, va, vb);
+  }
+  // scalar tail (fewer than 4 elements) handled by the first lanes of block 0
+  const int64_t t = n4 * 4 + (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (t < n) out[t] = f(HAS_A ? a[t] : 0.f, HAS_B ? b[t] : 0.f);
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <class F, bool HAS_A, bool HAS_B>
+int launch_ew(F f, float *out, const float *a, const float *b, int64_t n, hipStream_t s, const char *what) {
+  if (n <= 0) return 0;
+  int64_t n4 = n / 4;
+  if (!aligned16(out) || (HAS_A && !aligned16(a)) || (HAS_B && !aligned16(b))) n4 = 0;
+  const int64_t tail = n - n4 * 4;
+  int64_t blocks = (n4 + (int64_t)kThreads * kUnroll - 1) / ((int64_t)kThreads * kUnroll);
+  const int64_t cap = (int64_t)num_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  const int64_t tail_blocks = (tail + kThreads - 1) / kThreads;
+  if (blocks < tail_blocks) blocks = tail_blocks;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL((ew_kernel<F, HAS_A, HAS_B>), dim3((unsigned)blocks), dim3(kThreads), 0, s, f, out, a, b,
+                     n4, n);
+  return finish(s, what);
+}
+
+// out[i] = in[i % in_count]
+__global__ __launch_bounds__(kThreads) void broadcast_tail_kernel(const float *__restrict__ in, int in_count,
+                                                                 float *__restrict__ out, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+    out[i] = in[(int)(i % in_count)];
+}
+
+// out[n, c, inner] = in[c]; one float4 per lane when inner % 4 == 0
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void broadcast_channel_kernel(const float *__restrict__ in, int C,
+                                                                    int inner, float *__restrict__ out,
+                                                                    int64_t n_units) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  const int units_per_row = VEC ? inner / 4 : inner;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n_units; i += stride) {
+    const int c = (int)((i / units_per_row) % C);
+    const float v = in[c];
+    if (VEC) reinterpret_cast<float4 *>(out)[i] = make_float4(v, v, v, v);
+    else out[i] = v;
+  }
+}
+
+// out[i] = -s * y[i] / x[i] * dout[i]
+__global__ __launch_bounds__(kThreads) void cross_backward_kernel(const float *__restrict__ x,
+                                                                 const float *__restrict__ y,
+                                                                 const float *__restrict__ dout,
+                                                                 float *__restrict__ out, float s, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+    out[i] = y[i] * (-1.f) * s * (1.0f / x[i]) * dout[i];
+}
+
+// m = b1*m + (1-b1)*g ; v = b2*v + (1-b2)*g*g
+__global__ __launch_bounds__(kThreads) void adam_mv_kernel(float *m, float *v, const float *__restrict__ g,
+                                                          float b1, float b2, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
+    const float gi = g[i];
+    m[i] = m[i] * b1 + gi * (1.f - b1);
+    v[i] = v[i] * b2 + gi * gi * (1.f - b2);
+  }
+}
+
+// w -= lr * (m / (1-b1t)) / (sqrt(v / (1-b2t)) + e)
+__global__ __launch_bounds__(kThreads) void adam_kernel(float *w, const float *__restrict__ m,
+                                                       const float *__restrict__ v, float b1t, float b2t,
+                                                       float e, float lr, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+    w[i] = w[i] - lr * m[i] / (1.f - b1t) / (sqrtf(v[i] / (1.f - b2t)) + e);
+}
+
+// Fused multi-tensor SGD over a flat index space:
+// w[number[i]][offset[i]] -= lr * g[number[i]][offset[i]]
+__global__ __launch_bounds__(kThreads) void sgd_multi_kernel(float **w, float **g,
+                                                            const int *__restrict__ number,
+                                                            const int *__restrict__ offset, float lr,
+                                                            int count) {
+  const int stride = gridDim.x * kThreads;
+  for (int i = blockIdx.x * kThreads + threadIdx.x; i < count; i += stride) {
+    const int t = number[i], o = offset[i];
+    w[t][o] = w[t][o] - lr * g[t][o];
+  }
+}
+
+int grid_for(int64_t n) {
+  int64_t blocks = (n + kThreads - 1) / kThreads;
+  const int64_t cap = (int64_t)num_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  return blocks < 1 ? 1 : (int)blocks;
+}
+
+}  // namespace
+
+extern "C" int DLGpuArraySet(DLArrayHandle arr, float value, void **stream) {
+  TF_REQUIRE(on_gpu(arr), "array must live on the GPU");
+  hipStream_t s = stream_of(stream);
+  return launch_ew<OpSet, false, false>(OpSet{value}, (float *)arr->data, nullptr, nullptr, numel(arr), s,
+                                        "DLGpuArraySet");
+}
+
+extern "C" int DLGpuMatrixElementwiseAdd(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
+                                         void **stream) {
+  TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
+  return launch_ew<OpAdd, true, true>(OpAdd{}, (float *)out->data, (const float *)a->data,
+                                      (const float *)b->data, numel(out), stream_of(stream),
+                                      "DLGpuMatrixElementwiseAdd");
+}
+
+extern "C" int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle in, float val, DLArrayHandle out,
+                                                void **stream) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(in, out), "shape mismatch");
+  return launch_ew<OpAddC, true, false>(OpAddC{val}, (float *)out->data, (const float *)in->data, nullptr,
+                                        numel(out), stream_of(stream), "DLGpuMatrixElementwiseAddByConst");
+}
+
+extern "C" int DLGpuMatrixElementwiseMultiply(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
+                                              void **stream) {
+  TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
+  return launch_ew<OpMul, true, true>(OpMul{}, (float *)out->data, (const float *)a->data,
+                                      (const float *)b->data, numel(out), stream_of(stream),
+                                      "DLGpuMatrixElementwiseMultiply");
+}
+
+extern "C" int DLGpuMatrixMultiplyByConst(const DLArrayHandle in, float val, DLArrayHandle out,
+                                          void **stream) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(in, out), "shape mismatch");
+  return launch_ew<OpMulC, true, false>(OpMulC{val}, (float *)out->data, (const float *)in->data, nullptr,
+                                        numel(out), stream_of(stream), "DLGpuMatrixMultiplyByConst");
+}
+
+// The two stream-less entry points run on the legacy default stream, which is
+// ordered after all work already enqueued on the blocking streams created by
+// DLGpuCreatecudaStream and before any work enqueued on them later.
+extern "C" int DLGpuRelu(const DLArrayHandle in, DLArrayHandle out) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(in, out), "shape mismatch");
+  return launch_ew<OpRelu, true, false>(OpRelu{}, (float *)out->data, (const float *)in->data, nullptr,
+                                        numel(out), nullptr, "DLGpuRelu");
+}
+
+extern "C" int DLGpuReluGradient(const DLArrayHandle in, const DLArrayHandle grad, DLArrayHandle out) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(grad) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(in, out) && same_shape(grad, out), "shape mismatch");
+  return launch_ew<OpReluGrad, true, true>(OpReluGrad{}, (float *)out->data, (const float *)in->data,
+                                           (const float *)grad->data, numel(out), nullptr,
+                                           "DLGpuReluGradient");
+}
+
+extern "C" int DLGpuSgdUpdate(DLArrayHandle w, const DLArrayHandle g, float lr, void **stream) {
+  TF_REQUIRE(on_gpu(w) && on_gpu(g), "arrays must live on the GPU");
+  TF_REQUIRE(numel(w) == numel(g), "parameter and gradient differ in size");
+  return launch_ew<OpSgd, true, true>(OpSgd{lr}, (float *)w->data, (const float *)w->data,
+                                      (const float *)g->data, numel(w), stream_of(stream), "DLGpuSgdUpdate");
+}
+
+extern "C" int DLGpuCross(const DLArrayHandle x, const DLArrayHandle y, DLArrayHandle out, float b,
+                          void **stream) {
+  TF_REQUIRE(on_gpu(x) && on_gpu(y) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(numel(x) == numel(out) && numel(y) == numel(out), "shape mismatch");
+  return launch_ew<OpCross, true, true>(OpCross{b}, (float *)out->data, (const float *)x->data,
+                                        (const float *)y->data, numel(out), stream_of(stream), "DLGpuCross");
+}
+
+extern "C" int DLGpuCrossBackward(const DLArrayHandle x, const DLArrayHandle y, const DLArrayHandle dout,
+                                  DLArrayHandle out, float b, void **stream) {
+  TF_REQUIRE(on_gpu(x) && on_gpu(y) && on_gpu(dout) && on_gpu(out), "arrays must live on the GPU");
+  const int64_t n = numel(out);
+  TF_REQUIRE(numel(x) == n && numel(y) == n && numel(dout) == n, "shape mismatch");
+  hipStream_t s = stream_of(stream);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(cross_backward_kernel, dim3(grid_for(n)), dim3(kThreads), 0, s, (const float *)x->data,
+                     (const float *)y->data, (const float *)dout->data, (float *)out->data, b, n);
+  return finish(s, "DLGpuCrossBackward");
+}
+
+extern "C" int DLGpuBroadcastTo0(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  const int64_t in_count = numel(in), n = numel(out);
+  TF_REQUIRE(in_count > 0 && in_count <= INT32_MAX, "bad input size");
+  if (!(in->ndim == 1 && in->shape[0] == 1)) {
+    TF_REQUIRE(in->ndim <= out->ndim, "input has more dims than output");
+    for (int i = 0; i < in->ndim; ++i)
+      TF_REQUIRE(in->shape[in->ndim - 1 - i] == out->shape[out->ndim - 1 - i],
+                 "input must match the trailing dims of the output");
+  }
+  hipStream_t s = stream_of(stream);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(broadcast_tail_kernel, dim3(grid_for(n)), dim3(kThreads), 0, s, (const float *)in->data,
+                     (int)in_count, (float *)out->data, n);
+  return finish(s, "DLGpuBroadcastTo0");
+}
+
+extern "C" int DLGpuBroadcastTo1(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(in->ndim == 1 && out->ndim >= 2 && in->shape[0] == out->shape[1],
+             "input must be (C,) and output (N, C, ...)");
+  int64_t inner = 1;
+  for (int i = 2; i < out->ndim; ++i) inner *= out->shape[i];
+  const int64_t n = numel(out);
+  TF_REQUIRE(inner <= INT32_MAX, "inner extent too large");
+  hipStream_t s = stream_of(stream);
+  if (n == 0) return 0;
+  const int C = (int)out->shape[1];
+  if (inner % 4 == 0 && aligned16(out->data)) {
+    const int64_t units = n / 4;
+    hipLaunchKernelGGL(broadcast_channel_kernel<true>, dim3(grid_for(units)), dim3(kThreads), 0, s,
+                       (const float *)in->data, C, (int)inner, (float *)out->data, units);
+  } else {
+    hipLaunchKernelGGL(broadcast_channel_kernel<false>, dim3(grid_for(n)), dim3(kThreads), 0, s,
+                       (const float *)in->data, C, (int)inner, (float *)out->data, n);
+  }
+  return finish(s, "DLGpuBroadcastTo1");
+}
+
+extern "C" int DLGpuAdam_mv(DLArrayHandle m, DLArrayHandle v, const DLArrayHandle g, float b1, float b2,
+                            void **stream) {
+  TF_REQUIRE(on_gpu(m) && on_gpu(v) && on_gpu(g), "arrays must live on the GPU");
+  const int64_t n = numel(g);
+  TF_REQUIRE(numel(m) == n && numel(v) == n, "shape mismatch");
+  hipStream_t s = stream_of(stream);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(adam_mv_kernel, dim3(grid_for(n)), dim3(kThreads), 0, s, (float *)m->data,
+                     (float *)v->data, (const float *)g->data, b1, b2, n);
+  return finish(s, "DLGpuAdam_mv");
+}
+
+extern "C" int DLGpuAdam(DLArrayHandle w, const DLArrayHandle m, const DLArrayHandle v, float b1t, float b2t,
+                         float e, float lr, void **stream) {
+  TF_REQUIRE(on_gpu(w) && on_gpu(m) && on_gpu(v), "arrays must live on the GPU");
+  const int64_t n = numel(w);
+  TF_REQUIRE(numel(m) == n && numel(v) == n, "shape mismatch");
+  hipStream_t s = stream_of(stream);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(adam_kernel, dim3(grid_for(n)), dim3(kThreads), 0, s, (float *)w->data,
+                     (const float *)m->data, (const float *)v->data, b1t, b2t, e, lr, n);
+  return finish(s, "DLGpuAdam");
+}
+
+// ---- fused multi-tensor SGD --------------------------------------------------
+
+extern "C" int DLGpuGetIndextoVaribaleNumberCudaPointer(int *index_to_number, int *prefix, int count,
+                                                        void ***result) {
+  TF_REQUIRE(index_to_number && prefix && result && count >= 0, "bad arguments");
+  int *d_number = nullptr, *d_prefix = nullptr;
+  const size_t bytes = sizeof(int) * (size_t)(count > 0 ? count : 1);
+  TF_HIP(hipMalloc((void **)&d_number, bytes));
+  TF_HIP(hipMalloc((void **)&d_prefix, bytes));
+  TF_HIP(hipMemcpy(d_number, index_to_number, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
+  TF_HIP(hipMemcpy(d_prefix, prefix, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
+  *result = (void **)malloc(sizeof(void *) * 2);
+  (*result)[0] = d_number;
+  (*result)[1] = d_prefix;
+  return 0;
+}
+
+extern "C" int DLGpuGetN2CudaPointer(void **output, void **g, int number, void ****result) {
+  TF_REQUIRE(output && g && result && number >= 0, "bad arguments");
+  float **d_out = nullptr, **d_g = nullptr;
+  const size_t bytes = sizeof(float *) * (size_t)(number > 0 ? number : 1);
+  TF_HIP(hipMalloc((void **)&d_out, bytes));
+  TF_HIP(hipMalloc((void **)&d_g, bytes));
+  TF_HIP(hipMemcpy(d_out, output, sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
+  TF_HIP(hipMemcpy(d_g, g, sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
+  *result = (void ***)malloc(sizeof(void **) * 2);
+  (*result)[0] = (void **)d_out;
+  (*result)[1] = (void **)d_g;
+  return 0;
+}
+
+extern "C" int DLGpuSgd_o(void ****n2list, const void ***indexlist, const int count,
+                          const float learning_rate) {
+  TF_REQUIRE(n2list && *n2list && indexlist && *indexlist && count >= 0, "bad arguments");
+  if (count == 0) return 0;
+  // no stream argument: default stream, ordered against all created streams
+  hipLaunchKernelGGL(sgd_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, nullptr,
+                     (float **)((*n2list)[0]), (float **)((*n2list)[1]), (const int *)((*indexlist)[0]),
+                     (const int *)((*indexlist)[1]), learning_rate, count);
+  return finish(nullptr, "DLGpuSgd_o");
+}

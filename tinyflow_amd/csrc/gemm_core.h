@@ -1,0 +1,303 @@
+// fp32 MFMA tile engine shared by the matrix multiply and the three implicit-GEMM
+// convolutions (forward, grad-data, grad-filter).
+//
+//   D[m, n] = sum_k A(m, k) * B(k, n)
+//
+// One 256-lane workgroup (four wave64 waves in a 2 x 2 arrangement) owns a
+// BM x BN tile of D and walks the reduction in steps of BK = 16.  Operand tiles
+// are fetched with bounds-checked buffer loads (an out-of-range or padded
+// element is given an offset beyond the buffer and reads as zero, so tails and
+// convolution padding need no branches), staged through double-buffered LDS as
+// [k][m] / [k][n] planes, and consumed by v_mfma_f32_32x32x2_f32: per MFMA a
+// lane supplies A[m = lane%32][k = lane/32] and B[k = lane/32][n = lane%32],
+// and owns 16 accumulators D[8*(v/4) + 4*(lane/32) + v%4][lane%32].
+//
+// What differs between the four users is only how a tile element's address is
+// formed (the loader) and where an accumulator is written (the epilogue); both
+// are template policies defined next to their users.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace tf {
+namespace gemm {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 16;          // reduction depth of one LDS stage
+constexpr int THREADS = 256;    // four waves
+constexpr int LDS_PAD = 4;      // row padding of the LDS planes (floats)
+constexpr uint32_t OOB = 0x80000000u;  // byte offset that every buffer bound check rejects
+
+// Raw buffer resource over [base, base + bytes): loads past `bytes` return 0.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ inline float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+
+// Unsigned division by a runtime constant: q = (umulhi(n, mul) + n) >> shift,
+// exact for n < 2^31.
+struct FastDiv {
+  uint32_t d, mul, shift;
+  FastDiv() : d(1), mul(0), shift(0) {}
+  explicit FastDiv(uint32_t div) : d(div) {
+    uint32_t l = 0;
+    while ((1ull << l) < div) ++l;
+    shift = l;
+    mul = (uint32_t)((((1ull << l) - div) << 32) / div + 1);
+  }
+  __device__ inline uint32_t div(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
+  __device__ inline void divmod(uint32_t n, uint32_t &q, uint32_t &r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
+// ---- thread -> tile-element maps ---------------------------------------------
+// "Along" map: the 256 lanes run along the tile's m (or n) extent D, so that one
+// load instruction of a wave reads 64 consecutive m for a single, wave-uniform k.
+template <int D>
+struct AlongMap {
+  static_assert(D == 64 || D == 128 || D == 256, "tile extent");
+  static constexpr int KSTEP = THREADS / D;  // k rows covered per pass
+  static constexpr int EPT = BK / KSTEP;     // elements per thread per stage
+  int d_local;                               // position along the tile extent
+  int k_first;                               // wave-uniform
+  __device__ inline void init(int tid) {
+    d_local = tid % D;
+    k_first = __builtin_amdgcn_readfirstlane(tid / D);
+  }
+  __device__ inline int k_of(int e) const { return k_first + e * KSTEP; }
+};
+
+// "Across" map: 16 consecutive lanes run along k (the contiguous direction of
+// the operand in memory), the remaining 16 lane groups along the tile extent.
+template <int D>
+struct AcrossMap {
+  static_assert(D % 16 == 0, "tile extent");
+  static constexpr int DSTEP = THREADS / BK;  // 16
+  static constexpr int EPT = D / DSTEP;
+  int k_local;
+  int d_first;
+  __device__ inline void init(int tid) {
+    k_local = tid % BK;
+    d_first = tid / BK;
+  }
+  __device__ inline int d_of(int e) const { return d_first + e * DSTEP; }
+};
+
+// ---- plain row-major matrix operands -------------------------------------------
+// element(d, k) = base[k * ld + d]        (tile extent contiguous in memory)
+template <int D>
+struct PlainAlong {
+  using Map = AlongMap<D>;
+  static constexpr int EPT = Map::EPT;
+  const float *base;
+  uint32_t bytes;
+  int ld, d_extent, k_extent;
+
+  struct State {
+    Map map;
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t d_off;  // byte offset of this lane's d, or OOB
+  };
+  __device__ inline void init(State &st, int origin, int tid) const {
+    st.map.init(tid);
+    st.rsrc = make_rsrc(base, bytes);
+    const int d = origin + st.map.d_local;
+    st.d_off = d < d_extent ? (uint32_t)d * 4u : OOB;
+  }
+  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int k = k0 + st.map.k_of(e);
+      const uint32_t off = k < k_extent ? st.d_off + (uint32_t)k * (uint32_t)ld * 4u : OOB;
+      reg[e] = buf_load(st.rsrc, off | (st.d_off & OOB));
+    }
+  }
+  template <int LD>
+  __device__ inline void store(const State &st, float (*tile)[LD], const float (&reg)[EPT]) const {
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) tile[st.map.k_of(e)][st.map.d_local] = reg[e];
+  }
+};
+
+// element(d, k) = base[d * ld + k]        (reduction contiguous in memory)
+template <int D>
+struct PlainAcross {
+  using Map = AcrossMap<D>;
+  static constexpr int EPT = Map::EPT;
+  const float *base;
+  uint32_t bytes;
+  int ld, d_extent, k_extent;
+
+  struct State {
+    Map map;
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t row_off[EPT];  // byte offset of row d, or OOB
+  };
+  __device__ inline void init(State &st, int origin, int tid) const {
+    st.map.init(tid);
+    st.rsrc = make_rsrc(base, bytes);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int d = origin + st.map.d_of(e);
+      st.row_off[e] = d < d_extent ? (uint32_t)d * (uint32_t)ld * 4u : OOB;
+    }
+  }
+  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+    const int k = k0 + st.map.k_local;
+    const uint32_t k_off = k < k_extent ? (uint32_t)k * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) reg[e] = buf_load(st.rsrc, (st.row_off[e] + k_off) | ((st.row_off[e] | k_off) & OOB));
+  }
+  template <int LD>
+  __device__ inline void store(const State &st, float (*tile)[LD], const float (&reg)[EPT]) const {
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) tile[st.map.k_local][st.map.d_of(e)] = reg[e];
+  }
+};
+
+// ---- epilogue: plain row-major store ---------------------------------------------
+struct StoreRowMajor {
+  float *out;
+  int ld, m_extent, n_extent;
+  int64_t split_stride;  // elements between the outputs of consecutive k-splits
+  struct State {
+    float *base;
+  };
+  template <int TN>
+  __device__ inline void init(State &st, int /*n0*/, int /*lane*/, int split) const {
+    st.base = out + (int64_t)split * split_stride;
+  }
+  __device__ inline void store(const State &st, int m, int n, int /*j*/, float v) const {
+    if (m < m_extent && n < n_extent) st.base[(int64_t)m * ld + n] = v;
+  }
+};
+
+// ---- the kernel ----------------------------------------------------------------------
+// Work decomposition: gridDim.x = tiles_m * tiles_n * splits.  Hardware hands
+// consecutive workgroup ids to the 8 XCDs round-robin; the remap below gives
+// each XCD a contiguous range of logical tile ids, ordered m-fastest, so the
+// workgroups that share one B tile (the large, gathered operand) also share an
+// L2.  Every wave executes the same number of barriers and exits after its
+// epilogue; there is no data-dependent loop.
+template <int BM, int BN, class ALoader, class BLoader, class Epilogue>
+__global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const BLoader bl, const Epilogue ep,
+                                                      int k_extent, int k_per_split, int tiles_m, int tiles_n) {
+  constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  static_assert(TM >= 1 && TN >= 1, "tile too small for a 2x2 wave grid");
+  constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
+  __shared__ float As[2][BK][LDA];
+  __shared__ float Bs[2][BK][LDB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+
+  // XCD-aware logical id
+  const int nb = gridDim.x;
+  const int per_xcd = nb >> 3;
+  int logical = blockIdx.x;
+  if (logical < (per_xcd << 3)) logical = (logical & 7) * per_xcd + (logical >> 3);
+  const int tm = logical % tiles_m;
+  const int rest = logical / tiles_m;
+  const int tn = rest % tiles_n;
+  const int split = rest / tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int k_begin = split * k_per_split;
+  int k_end = k_begin + k_per_split;
+  if (k_end > k_extent) k_end = k_extent;
+
+  typename ALoader::State sa;
+  typename BLoader::State sb;
+  al.init(sa, m0, tid);
+  bl.init(sb, n0, tid);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  float ra[ALoader::EPT], rb[BLoader::EPT];
+  if (k_begin < k_end) {
+    al.load(sa, k_begin, ra);
+    bl.load(sb, k_begin, rb);
+    al.template store<LDA>(sa, As[0], ra);
+    bl.template store<LDB>(sb, Bs[0], rb);
+  }
+  __syncthreads();
+
+  const int lrow = lane >> 5;   // which of the two k of an MFMA this lane feeds
+  const int lcol = lane & 31;
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+    const bool has_next = k0 + BK < k_end;
+    if (has_next) {
+      al.load(sa, k0 + BK, ra);
+      bl.load(sb, k0 + BK, rb);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK / 2; ++kk) {
+      const int krow = 2 * kk + lrow;
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = As[buf][krow][wm * WM + 32 * i + lcol];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = Bs[buf][krow][wn * WN + 32 * j + lcol];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (has_next) {
+      al.template store<LDA>(sa, As[buf ^ 1], ra);
+      bl.template store<LDB>(sb, Bs[buf ^ 1], rb);
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  typename Epilogue::State se;
+  ep.template init<TN>(se, n0 + wn * WN, lane, split);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * lrow + (v & 3);
+        const int n = n0 + wn * WN + 32 * j + lcol;
+        ep.store(se, m, n, j, acc[i][j][v]);
+      }
+}
+
+// Host-side launch geometry shared by the users.
+struct Geometry {
+  int tiles_m, tiles_n, splits, k_per_split;
+  unsigned blocks() const { return (unsigned)(tiles_m * tiles_n * splits); }
+};
+inline Geometry make_geometry(int M, int N, int K, int bm, int bn, int splits) {
+  Geometry g;
+  g.tiles_m = (M + bm - 1) / bm;
+  g.tiles_n = (N + bn - 1) / bn;
+  if (splits < 1) splits = 1;
+  int kps = ((K + splits - 1) / splits + BK - 1) / BK * BK;
+  if (kps < BK) kps = BK;
+  g.k_per_split = kps;
+  g.splits = (K + kps - 1) / kps;
+  if (g.splits < 1) g.splits = 1;
+  return g;
+}
+
+}  // namespace gemm
+}  // namespace tf

@@ -1,0 +1,142 @@
+// Internal helpers shared by the HIP sources of libc_runtime_api.so.
+// Nothing here is part of the C-ABI; the exported surface is include/c_runtime_api.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+#include "c_runtime_api.h"
+
+namespace tf {
+
+// ---- device scratch / array storage: caching allocator (runtime.hip) -------
+// Blocks are recycled by size; a freed block may still be read by kernels that
+// are already enqueued, which is safe because every consumer is ordered after
+// them (same stream, or cross-stream wait inserted by DLArrayCopyFromTo).
+void *device_alloc(size_t bytes);  // nullptr when the device (or the cap) is exhausted
+void device_free(void *p);
+void *pinned_alloc(size_t bytes);
+void pinned_free(void *p);
+
+// ---- streams ----------------------------------------------------------------
+hipStream_t stream_of(void **cell);      // cell written by DLGpuCreatecudaStream; NULL -> default stream
+bool sync_every_op();                    // TINYFLOW_SYNC_EVERY_OP=1
+int finish(hipStream_t s, const char *what);  // launch-error check (+ optional sync)
+
+// ---- small host utilities -----------------------------------------------------
+inline int64_t numel(const DLArray *a) {
+  int64_t n = 1;
+  for (int i = 0; i < a->ndim; ++i) n *= a->shape[i];
+  return n;
+}
+inline bool same_shape(const DLArray *a, const DLArray *b) {
+  if (a->ndim != b->ndim) return false;
+  for (int i = 0; i < a->ndim; ++i)
+    if (a->shape[i] != b->shape[i]) return false;
+  return true;
+}
+inline bool on_gpu(const DLArray *a) { return a && a->data && a->ctx.device_type == kGPU; }
+
+inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+// Number of compute units of the current device (256 on MI355X).
+int num_cus();
+
+}  // namespace tf
+
+#define TF_REQUIRE(cond, ...)                                  \
+  do {                                                         \
+    if (!(cond)) {                                             \
+      fprintf(stderr, "[tinyflow_amd] %s: ", __func__);        \
+      fprintf(stderr, __VA_ARGS__);                            \
+      fprintf(stderr, "\n");                                   \
+      return -1;                                               \
+    }                                                          \
+  } while (0)
+
+#define TF_HIP(expr)                                                          \
+  do {                                                                        \
+    hipError_t _e = (expr);                                                   \
+    if (_e != hipSuccess) {                                                   \
+      fprintf(stderr, "[tinyflow_amd] %s: %s failed: %s\n", __func__, #expr,  \
+              hipGetErrorString(_e));                                         \
+      return -1;                                                              \
+    }                                                                         \
+  } while (0)
+
+// Opaque descriptor structs placed behind the `void ***list` arguments.
+namespace tf {
+
+constexpr int kMagicConv = 0x74664376;    // 'tfCv'
+constexpr int kMagicPool = 0x7466506c;    // 'tfPl'
+constexpr int kMagicAct = 0x74664163;     // 'tfAc'
+constexpr int kMagicBN = 0x7466424e;      // 'tfBN'
+constexpr int kMagicReduce = 0x74665264;  // 'tfRd'
+constexpr int kMagicHandle = 0x74664864;  // 'tfHd'
+
+struct Handle {
+  int magic;
+  hipStream_t stream;
+};
+
+struct ConvDesc {
+  int magic;
+  int N, C, H, W;      // input
+  int K, R, S;         // filter (K output channels, C input channels)
+  int P, Q;            // output spatial
+  int pad_h, pad_w, u, v;
+  // device tables built lazily on first use (conv.hip); indexed by the
+  // reduction index of each implicit GEMM
+  int *fwd_tab;        // [C*R*S] x 2: element offset c*H*W + r*W + s, packed (r<<16|s)
+  int *dgrad_tab;      // [K*R*S] x 2: element offset k*P*Q - r*Q - s, packed taps
+};
+
+struct PoolDesc {
+  int magic;
+  int N, C, H, W, P, Q;
+  int mode;            // 0 max, 1 mean (count includes padding)
+  int pad_h, pad_w, u, v, fh, fw;
+};
+
+struct ActDesc {
+  int magic;
+  int mode;
+  int64_t n, inner;    // n instances of `inner` = c*h*w elements
+};
+
+struct BNDesc {
+  int magic;
+  int mode;            // 0 per-activation, 1 spatial
+  int N, C, HW;        // x viewed as [N, C, HW]
+  int64_t stat_count;  // C*HW (per-activation) or C (spatial)
+};
+
+struct ReduceDesc {
+  int magic;
+  int ndim;
+  int in[5];
+  int out[5];
+};
+
+template <class T>
+inline T *desc_from_list(void ***list, int magic) {
+  if (!list || !*list) return nullptr;
+  T *d = reinterpret_cast<T *>((*list)[0]);
+  if (!d || d->magic != magic) return nullptr;
+  return d;
+}
+
+}  // namespace tf
+
+// Cross-file kernel launchers.
+namespace tf {
+// out[i] = sum_s partial[s * count + i] in split order (matmul.hip)
+int launch_split_sum(const float *partial, float *out, int64_t count, int splits, hipStream_t s);
+int choose_splits(int tiles, int K, int min_k);
+// row softmax and its backward over [rows, cols] (reduce.hip)
+int launch_softmax_rows(const float *in, float *out, int64_t rows, int cols, hipStream_t s);
+int launch_softmax_rows_backward(const float *y, const float *dy, float *dx, int64_t rows, int cols,
+                                 hipStream_t s);
+}  // namespace tf

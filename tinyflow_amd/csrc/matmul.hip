@@ -1,0 +1,131 @@
+// DLGpuMatrixMultiply: C = op(A) * op(B) on the fp32 MFMA tile engine.
+//
+// Replaces the cublasSgemm call of the reference (src/gpu_op.cu:1166-1199).
+// The same entry point serves the forward product and both gradients the
+// autodiff emits for it (dA = dY * B^T, dB = A^T * dY,
+// pycode/tinyflow/autodiff.py:477-506), so all four transpose combinations are
+// first-class: a transposed operand only changes which loader reads it.
+//
+// Skinny problems (few output tiles, long reduction - e.g. a batch-32 fully
+// connected layer) are split along k into partial products that a second,
+// fixed-order pass adds up, so results do not depend on scheduling.
+#include "gemm_core.h"
+#include "internal.h"
+
+using namespace tf;
+using namespace tf::gemm;
+
+namespace {
+
+// out[i] = sum_s partial[s * count + i], splits added in index order
+__global__ __launch_bounds__(256) void split_sum_kernel(const float *__restrict__ partial,
+                                                       float *__restrict__ out, int64_t count, int splits) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += stride) {
+    float s = partial[i];
+    for (int k = 1; k < splits; ++k) s += partial[(int64_t)k * count + i];
+    out[i] = s;
+  }
+}
+
+template <int BM, int BN, class AL, class BL>
+void launch(const AL &al, const BL &bl, const StoreRowMajor &ep, int K, const Geometry &g, hipStream_t s) {
+  hipLaunchKernelGGL((gemm_kernel<BM, BN, AL, BL, StoreRowMajor>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl,
+                     ep, K, g.k_per_split, g.tiles_m, g.tiles_n);
+}
+
+template <int BM, int BN>
+void dispatch(const float *A, bool tA, int lda, uint32_t a_bytes, const float *B, bool tB, int ldb,
+              uint32_t b_bytes, const StoreRowMajor &ep, int M, int N, int K, const Geometry &g, hipStream_t s) {
+  if (!tA && !tB) {
+    PlainAcross<BM> al{A, a_bytes, lda, M, K};
+    PlainAlong<BN> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN>(al, bl, ep, K, g, s);
+  } else if (tA && !tB) {
+    PlainAlong<BM> al{A, a_bytes, lda, M, K};
+    PlainAlong<BN> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN>(al, bl, ep, K, g, s);
+  } else if (!tA && tB) {
+    PlainAcross<BM> al{A, a_bytes, lda, M, K};
+    PlainAcross<BN> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN>(al, bl, ep, K, g, s);
+  } else {
+    PlainAlong<BM> al{A, a_bytes, lda, M, K};
+    PlainAcross<BN> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN>(al, bl, ep, K, g, s);
+  }
+}
+
+}  // namespace
+
+namespace tf {
+
+int launch_split_sum(const float *partial, float *out, int64_t count, int splits, hipStream_t s) {
+  int64_t blocks = (count + 255) / 256;
+  const int64_t cap = (int64_t)num_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, s, partial, out, count, splits);
+  return 0;
+}
+
+// Number of k-splits that brings `tiles` output tiles up to about two
+// workgroups per CU without making a split shorter than `min_k` reduction steps.
+int choose_splits(int tiles, int K, int min_k) {
+  const int target = 2 * num_cus();
+  if (tiles >= target) return 1;
+  int splits = (target + tiles - 1) / tiles;
+  const int max_splits = K / min_k;
+  if (splits > max_splits) splits = max_splits;
+  return splits < 1 ? 1 : splits;
+}
+
+}  // namespace tf
+
+extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
+                                   bool transposeB, DLArrayHandle matC, void **handle, void **stream) {
+  (void)handle;
+  TF_REQUIRE(on_gpu(matA) && on_gpu(matB) && on_gpu(matC), "arrays must live on the GPU");
+  TF_REQUIRE(matA->ndim == 2 && matB->ndim == 2 && matC->ndim == 2, "operands must be 2-D");
+  const int64_t M = matA->shape[transposeA ? 1 : 0], K = matA->shape[transposeA ? 0 : 1];
+  const int64_t Kb = matB->shape[transposeB ? 1 : 0], N = matB->shape[transposeB ? 0 : 1];
+  TF_REQUIRE(K == Kb, "inner dimensions differ (%lld vs %lld)", (long long)K, (long long)Kb);
+  TF_REQUIRE(matC->shape[0] == M && matC->shape[1] == N, "output must be %lld x %lld", (long long)M,
+             (long long)N);
+  const int64_t a_bytes = numel(matA) * 4, b_bytes = numel(matB) * 4;
+  TF_REQUIRE(a_bytes < (1ll << 31) && b_bytes < (1ll << 31) && M * N < (1ll << 31),
+             "operand larger than 2 GiB is not supported");
+  hipStream_t s = stream_of(stream);
+  if (M == 0 || N == 0) return 0;
+  if (K == 0) return DLGpuArraySet(matC, 0.f, stream);
+
+  const int lda = (int)matA->shape[1], ldb = (int)matB->shape[1];
+  const bool big = M > 64 && N > 64 && cdiv(M, 128) * cdiv(N, 128) >= num_cus();
+  const int bm = big ? 128 : 64, bn = big ? 128 : 64;
+  const int tiles = cdiv(M, bm) * cdiv(N, bn);
+  const int splits = choose_splits(tiles, (int)K, 8 * BK);
+  Geometry g = make_geometry((int)M, (int)N, (int)K, bm, bn, splits);
+
+  float *dst = (float *)matC->data;
+  float *partial = nullptr;
+  if (g.splits > 1) {
+    partial = (float *)device_alloc((size_t)g.splits * M * N * sizeof(float));
+    if (!partial) {  // no scratch: fall back to one pass over the whole reduction
+      g = make_geometry((int)M, (int)N, (int)K, bm, bn, 1);
+    } else {
+      dst = partial;
+    }
+  }
+  StoreRowMajor ep{dst, (int)N, (int)M, (int)N, M * N};
+  if (big)
+    dispatch<128, 128>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
+                       transposeB, ldb, (uint32_t)b_bytes, ep, (int)M, (int)N, (int)K, g, s);
+  else
+    dispatch<64, 64>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
+                     transposeB, ldb, (uint32_t)b_bytes, ep, (int)M, (int)N, (int)K, g, s);
+  if (partial) {
+    launch_split_sum(partial, (float *)matC->data, M * N, g.splits, s);
+    device_free(partial);
+  }
+  return finish(s, "DLGpuMatrixMultiply");
+}

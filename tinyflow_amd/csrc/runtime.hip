@@ -1,0 +1,395 @@
+// Thin HIP device API behind DLArrayAlloc / DLArrayFree / DLArrayCopyFromTo and
+// the stream / handle factories.
+//
+// Replaces the reference's DeviceAPIManager + CUDADeviceAPI + CPUDeviceAPI
+// (src/c_runtime_api.cc:21-164, src/cuda_device_api.cc:22-81,
+// src/cpu_device_api.cc:12-36).  Differences that are deliberate:
+//   * device and pinned-host storage come from a caching allocator, so the
+//     executor's allocate-per-node-per-step pattern (pycode/tinyflow/autodiff.py:2778)
+//     costs a map lookup instead of a hipMalloc/hipFree pair;
+//   * ops do not block the host; copies order themselves after enqueued work.
+#include "internal.h"
+
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace tf {
+namespace {
+
+struct StreamRec {
+  hipStream_t stream;
+  hipEvent_t event;  // reusable marker for cross-stream ordering
+};
+
+struct Runtime {
+  std::mutex mu;
+  // caching allocator state (one per memory kind)
+  struct Pool {
+    std::multimap<size_t, void *> free_blocks;      // size -> block
+    std::unordered_map<void *, size_t> block_size;  // every block obtained from HIP
+    size_t reserved = 0;                            // bytes held from HIP (in use + cached)
+  };
+  Pool dev, host;
+  size_t dev_limit = 0;  // 0 = unlimited; TINYFLOW_GPU_MEM_LIMIT_MB
+  std::vector<StreamRec> streams;
+  bool sync_ops = false;
+  int cus = 0;
+  bool inited = false;
+
+  void init() {
+    if (inited) return;
+    inited = true;
+    if (const char *e = getenv("TINYFLOW_GPU_MEM_LIMIT_MB")) dev_limit = (size_t)atoll(e) << 20;
+    if (const char *e = getenv("TINYFLOW_SYNC_EVERY_OP")) sync_ops = atoi(e) != 0;
+  }
+};
+
+Runtime &rt() {
+  static Runtime *r = new Runtime();  // leaked on purpose: arrays may be freed during interpreter exit
+  return *r;
+}
+
+size_t round_size(size_t bytes) {
+  if (bytes == 0) bytes = 1;
+  const size_t q = bytes < (1u << 20) ? 512 : (size_t)1 << 16;  // 512 B below 1 MiB, 64 KiB above
+  return (bytes + q - 1) / q * q;
+}
+
+// Give every cached block of `p` back to HIP.  hipFree waits for the device, so
+// blocks still referenced by enqueued kernels are safe to release.
+void release_cached(Runtime::Pool &p, bool device) {
+  for (auto &kv : p.free_blocks) {
+    if (device) (void)hipFree(kv.second); else (void)hipHostFree(kv.second);
+    p.reserved -= kv.first;
+    p.block_size.erase(kv.second);
+  }
+  p.free_blocks.clear();
+}
+
+void *pool_alloc(Runtime::Pool &p, size_t bytes, bool device, size_t limit) {
+  const size_t want = round_size(bytes);
+  auto it = p.free_blocks.lower_bound(want);
+  // accept a cached block when it wastes at most 1/8 of its size
+  if (it != p.free_blocks.end() && it->first - want <= it->first / 8) {
+    void *ptr = it->second;
+    p.free_blocks.erase(it);
+    return ptr;
+  }
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    if (limit == 0 || p.reserved + want <= limit) {
+      void *ptr = nullptr;
+      hipError_t e = device ? hipMalloc(&ptr, want) : hipHostMalloc(&ptr, want, hipHostMallocDefault);
+      if (e == hipSuccess && ptr) {
+        p.block_size[ptr] = want;
+        p.reserved += want;
+        return ptr;
+      }
+      (void)hipGetLastError();  // clear the sticky out-of-memory error
+    }
+    if (attempt == 0) {
+      if (p.free_blocks.empty()) break;
+      release_cached(p, device);
+    }
+  }
+  return nullptr;
+}
+
+void pool_free(Runtime::Pool &p, void *ptr) {
+  if (!ptr) return;
+  auto it = p.block_size.find(ptr);
+  if (it == p.block_size.end()) return;  // not ours (e.g. a borrowed numpy buffer)
+  p.free_blocks.emplace(it->second, ptr);
+}
+
+}  // namespace
+
+void *device_alloc(size_t bytes) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  r.init();
+  return pool_alloc(r.dev, bytes, true, r.dev_limit);
+}
+void device_free(void *p) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  pool_free(r.dev, p);
+}
+void *pinned_alloc(size_t bytes) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  r.init();
+  return pool_alloc(r.host, bytes, false, 0);
+}
+void pinned_free(void *p) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  pool_free(r.host, p);
+}
+
+hipStream_t stream_of(void **cell) { return cell ? reinterpret_cast<hipStream_t>(*cell) : nullptr; }
+
+bool sync_every_op() {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  r.init();
+  return r.sync_ops;
+}
+
+int finish(hipStream_t s, const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fprintf(stderr, "[tinyflow_amd] %s: launch failed: %s\n", what, hipGetErrorString(e));
+    return -1;
+  }
+  if (sync_every_op()) {
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) {
+      fprintf(stderr, "[tinyflow_amd] %s: %s\n", what, hipGetErrorString(e));
+      return -1;
+    }
+  }
+  return 0;
+}
+
+int num_cus() {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  if (r.cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      r.cus = n;
+    else
+      r.cus = 256;
+  }
+  return r.cus;
+}
+
+}  // namespace tf
+
+using namespace tf;
+
+// ------------------------------------------------------------------ arrays
+
+static size_t array_bytes(const DLArray *a) { return (size_t)numel(a) * sizeof(float); }
+
+extern "C" int DLArrayAlloc(const index_t *shape, index_t ndim_in, DLContext ctx,
+                            DLArrayHandle *out, int *memorytoSaving) {
+  // The binding passes ndim as a 32-bit c_int although the prototype says int64:
+  // only the low word is defined.
+  const int ndim = (int)(ndim_in & 0xffffffff);
+  TF_REQUIRE(shape && out && ndim >= 0 && ndim <= 8, "bad arguments (ndim=%d)", ndim);
+  TF_REQUIRE(ctx.device_type == kCPU || ctx.device_type == kGPU, "unknown device type %d",
+             (int)ctx.device_type);
+  size_t bytes = sizeof(float);
+  for (int i = 0; i < ndim; ++i) {
+    TF_REQUIRE(shape[i] >= 0, "negative extent");
+    bytes *= (size_t)shape[i];
+  }
+  void *data = nullptr;
+  if (ctx.device_type == kGPU) {
+    TF_HIP(hipSetDevice(ctx.device_id));
+    data = device_alloc(bytes);
+  } else {
+    data = pinned_alloc(bytes);
+  }
+  if (!data) {
+    // out-of-memory convention of the reference: report the size, leave *out alone
+    if (memorytoSaving) *memorytoSaving = (int)bytes;
+    return 0;
+  }
+  DLArray *arr = new DLArray();
+  arr->data = data;
+  arr->ctx = ctx;
+  arr->ndim = ndim;
+  arr->shape = new int64_t[ndim > 0 ? ndim : 1];
+  for (int i = 0; i < ndim; ++i) arr->shape[i] = shape[i];
+  *out = arr;
+  return 0;
+}
+
+extern "C" int DLArrayFree(DLArrayHandle handle) {
+  if (!handle) return 0;
+  if (handle->data) {
+    if (handle->ctx.device_type == kGPU) device_free(handle->data);
+    else pinned_free(handle->data);
+  }
+  delete[] handle->shape;
+  delete handle;
+  return 0;
+}
+
+namespace {
+
+hipMemcpyKind copy_kind(const DLArray *from, const DLArray *to) {
+  const bool fg = from->ctx.device_type == kGPU, tg = to->ctx.device_type == kGPU;
+  if (fg && tg) return hipMemcpyDeviceToDevice;
+  if (fg) return hipMemcpyDeviceToHost;
+  if (tg) return hipMemcpyHostToDevice;
+  return hipMemcpyHostToHost;
+}
+
+// Make `s` wait for everything already enqueued on the other streams created
+// through DLGpuCreatecudaStream.
+int wait_for_other_streams(hipStream_t s) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  for (auto &rec : r.streams) {
+    if (rec.stream == s) continue;
+    TF_HIP(hipEventRecord(rec.event, rec.stream));
+    TF_HIP(hipStreamWaitEvent(s, rec.event, 0));
+  }
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
+  TF_REQUIRE(from && to && from->data && to->data, "null array");
+  const size_t bytes = array_bytes(from);
+  TF_REQUIRE(bytes == array_bytes(to), "size mismatch (%zu vs %zu bytes)", bytes, array_bytes(to));
+  const hipMemcpyKind kind = copy_kind(from, to);
+  if (bytes == 0) return 0;
+  if (kind == hipMemcpyHostToHost) {
+    memcpy(to->data, from->data, bytes);
+    return 0;
+  }
+  if (stream == nullptr) {
+    // synchronous form: everything enqueued so far is finished first, so the
+    // caller sees the results of all preceding ops
+    TF_HIP(hipDeviceSynchronize());
+    TF_HIP(hipMemcpy(to->data, from->data, bytes, kind));
+    if (kind == hipMemcpyDeviceToDevice) TF_HIP(hipDeviceSynchronize());
+    return 0;
+  }
+  hipStream_t s = stream_of(reinterpret_cast<void **>(stream));
+  if (wait_for_other_streams(s) != 0) return -1;
+  TF_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, s));
+  // Host memory must be readable / reusable on return.  A device-to-device copy
+  // is only ever observed by later stream-ordered work, so it stays asynchronous.
+  if (kind != hipMemcpyDeviceToDevice || sync_every_op()) TF_HIP(hipStreamSynchronize(s));
+  return 0;
+}
+
+extern "C" int getInt(int *intp) { return intp ? *intp : 0; }
+
+// ----------------------------------------------------- streams and handles
+
+extern "C" int DLGpuCreatecudaStream(void **cell) {
+  TF_REQUIRE(cell, "null cell");
+  hipStream_t s = nullptr;
+  // default priority, blocking with respect to the legacy default stream: the
+  // stream-less entry points (DLGpuRelu, DLGpuReluGradient) launch on the
+  // default stream and are ordered against every stream created here.
+  TF_HIP(hipStreamCreateWithFlags(&s, hipStreamDefault));
+  hipEvent_t ev = nullptr;
+  TF_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  {
+    Runtime &r = rt();
+    std::lock_guard<std::mutex> g(r.mu);
+    r.init();
+    r.streams.push_back({s, ev});
+  }
+  *cell = s;
+  return 0;
+}
+
+extern "C" int DLGpuDestroycudaStream(void **cell) {
+  TF_REQUIRE(cell, "null cell");
+  hipStream_t s = reinterpret_cast<hipStream_t>(*cell);
+  hipEvent_t ev = nullptr;
+  bool found = false;
+  {
+    Runtime &r = rt();
+    std::lock_guard<std::mutex> g(r.mu);
+    for (size_t i = 0; i < r.streams.size(); ++i)
+      if (r.streams[i].stream == s) {
+        ev = r.streams[i].event;
+        r.streams.erase(r.streams.begin() + i);
+        found = true;
+        break;
+      }
+  }
+  TF_REQUIRE(found, "not a stream created by DLGpuCreatecudaStream");
+  TF_HIP(hipStreamSynchronize(s));
+  TF_HIP(hipEventDestroy(ev));
+  TF_HIP(hipStreamDestroy(s));
+  *cell = nullptr;
+  return 0;
+}
+
+static int make_handle(void **cell, void **stream_cell) {
+  TF_REQUIRE(cell, "null cell");
+  Handle *h = new Handle();
+  h->magic = kMagicHandle;
+  h->stream = stream_of(stream_cell);
+  *cell = h;
+  return 0;
+}
+static int drop_handle(void **cell) {
+  TF_REQUIRE(cell && *cell, "null handle");
+  Handle *h = reinterpret_cast<Handle *>(*cell);
+  TF_REQUIRE(h->magic == kMagicHandle, "not a handle created by this library");
+  h->magic = 0;
+  delete h;
+  *cell = nullptr;
+  return 0;
+}
+
+extern "C" int DLGpuCreatecudnnHandle(void **handle, void **stream) { return make_handle(handle, stream); }
+extern "C" int DLGpuDestroycudnnHandle(void **handle) { return drop_handle(handle); }
+extern "C" int DLGpuCreatecublasHandle(void **handle, void **stream) { return make_handle(handle, stream); }
+extern "C" int DLGpuDestroycublasHandle(void **handle) { return drop_handle(handle); }
+
+// ---------------------------------------------------------------- testPcie
+
+// Host<->device bandwidth probe: 16 MiB each way, pageable and pinned, with a
+// byte-exact round-trip check (reference: src/gpu_op.cu:4915-5005).
+extern "C" int testPcie() {
+  const size_t bytes = (size_t)16 << 20;
+  const size_t n = bytes / sizeof(float);
+  float *pageable_a = (float *)malloc(bytes), *pageable_b = (float *)malloc(bytes);
+  float *pinned_a = nullptr, *pinned_b = nullptr, *dev = nullptr;
+  TF_REQUIRE(pageable_a && pageable_b, "host malloc failed");
+  TF_HIP(hipHostMalloc((void **)&pinned_a, bytes, hipHostMallocDefault));
+  TF_HIP(hipHostMalloc((void **)&pinned_b, bytes, hipHostMallocDefault));
+  TF_HIP(hipMalloc((void **)&dev, bytes));
+  for (size_t i = 0; i < n; ++i) pageable_a[i] = pinned_a[i] = (float)i;
+  hipEvent_t t0, t1;
+  TF_HIP(hipEventCreate(&t0));
+  TF_HIP(hipEventCreate(&t1));
+  struct Case { const char *name; float *src, *dst; } cases[2] = {
+      {"pageable", pageable_a, pageable_b}, {"pinned", pinned_a, pinned_b}};
+  int rc = 0;
+  for (auto &c : cases) {
+    float ms = 0.f;
+    memset(c.dst, 0, bytes);
+    TF_HIP(hipEventRecord(t0, nullptr));
+    TF_HIP(hipMemcpy(dev, c.src, bytes, hipMemcpyHostToDevice));
+    TF_HIP(hipEventRecord(t1, nullptr));
+    TF_HIP(hipEventSynchronize(t1));
+    TF_HIP(hipEventElapsedTime(&ms, t0, t1));
+    printf("%s host->device: %.2f GB/s\n", c.name, bytes * 1e-6 / ms);
+    TF_HIP(hipEventRecord(t0, nullptr));
+    TF_HIP(hipMemcpy(c.dst, dev, bytes, hipMemcpyDeviceToHost));
+    TF_HIP(hipEventRecord(t1, nullptr));
+    TF_HIP(hipEventSynchronize(t1));
+    TF_HIP(hipEventElapsedTime(&ms, t0, t1));
+    printf("%s device->host: %.2f GB/s\n", c.name, bytes * 1e-6 / ms);
+    if (memcmp(c.src, c.dst, bytes) != 0) {
+      printf("%s round trip MISMATCH\n", c.name);
+      rc = -1;
+    }
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  (void)hipFree(dev);
+  (void)hipHostFree(pinned_a);
+  (void)hipHostFree(pinned_b);
+  free(pageable_a);
+  free(pageable_b);
+  return rc;
+}
