@@ -1,0 +1,137 @@
+"""GPU parity of conv2d forward / grad-data / grad-filter against the oracle.
+
+Tolerance: rtol 1e-3 / atol 1e-5 relative to a float64 evaluation of the
+oracle (the bound BASELINE.json states for conv gradients); the cases cover every
+filter/stride/padding family of the LeNet, VGG-16 and ResNet-50 configs at
+reduced batch or spatial size, plus ragged sizes that exercise every tile tail.
+"""
+import numpy as np
+import pytest
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+# (N, C, H, W, K, R, S, padding, u, v)
+CONV_CASES = [
+    # reference tests/autodiff_test.py:335-343: x (5,1,4,4), w (1,1,3,3)
+    (5, 1, 4, 4, 1, 3, 3, "VALID", 1, 1),
+    (5, 1, 4, 4, 1, 3, 3, "SAME", 1, 1),
+    # LeNet-5
+    (64, 1, 28, 28, 6, 5, 5, "SAME", 1, 1),
+    (64, 6, 14, 14, 16, 5, 5, "VALID", 1, 1),
+    # VGG-style 3x3 pad 1
+    (2, 3, 32, 32, 64, 3, 3, "SAME", 1, 1),
+    (2, 64, 28, 28, 128, 3, 3, "SAME", 1, 1),
+    # ResNet-50 families (batch 4)
+    (4, 3, 64, 64, 64, 7, 7, "SAME", 2, 2),      # stem 7x7 s2 p3
+    (4, 64, 56, 56, 64, 1, 1, "VALID", 1, 1),    # 1x1 s1
+    (4, 64, 56, 56, 256, 1, 1, "VALID", 1, 1),
+    (4, 256, 56, 56, 128, 1, 1, "VALID", 2, 2),  # 1x1 s2 (first conv of a stage)
+    (4, 256, 56, 56, 512, 1, 1, "VALID", 2, 2),  # 1x1 s2 shortcut
+    (4, 128, 28, 28, 128, 3, 3, "SAME", 1, 1),
+    (4, 512, 7, 7, 512, 3, 3, "SAME", 1, 1),
+    (4, 2048, 7, 7, 512, 1, 1, "VALID", 1, 1),
+    (4, 1024, 14, 14, 2048, 1, 1, "VALID", 2, 2),
+    # ragged everything: odd sizes, non-square filter, different strides
+    (3, 5, 13, 11, 7, 3, 2, "SAME", 1, 1),
+    (2, 9, 17, 19, 70, 3, 3, "VALID", 2, 2),     # strided 3x3 (generic grad-data path)
+    (2, 4, 15, 15, 5, 5, 5, "SAME", 3, 2),
+    (1, 1, 1, 1, 1, 1, 1, "VALID", 1, 1),
+    (2, 3, 9, 9, 4, 1, 1, "VALID", 2, 2),        # 1x1 s2 on an odd extent
+    (2, 130, 6, 6, 67, 1, 1, "VALID", 3, 3),
+]
+
+
+def _gpu(a, rt):
+    from tinyflow_amd import ndarray
+    return ndarray.array(np.asarray(a, dtype=np.float32), rt.ctx)
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_conv_forward_and_gradients(rt, case):
+    from tinyflow_amd import gpu_op, ndarray
+    N, C, H, W, K, R, S, padding, u, v = case
+    rng = np.random.RandomState(abs(hash(case)) % (2 ** 31))
+    x = rng.normal(0, 1, (N, C, H, W)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(2.0 / (C * R * S)), (K, C, R, S)).astype(np.float32)
+    pad_h, pad_w = O.conv_pad(R, padding), O.conv_pad(S, padding)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", padding, u, v)
+    P, Q = O.conv_out_extent(H, R, pad_h, u), O.conv_out_extent(W, S, pad_w, v)
+    assert out_shape == (N, K, P, Q)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+
+    x64, w64, dy64 = x.astype(np.float64), w.astype(np.float64), dy.astype(np.float64)
+    y_ref = O.conv2d_forward(x64, w64, pad_h, pad_w, u, v)
+    dx_ref = O.conv2d_backward_data(dy64, w64, x.shape, pad_h, pad_w, u, v)
+    dw_ref = O.conv2d_backward_filter(x64, dy64, w.shape, pad_h, pad_w, u, v)
+
+    gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
+    gy = ndarray.empty(out_shape, rt.ctx)
+    gdx = ndarray.empty(x.shape, rt.ctx)
+    gdw = ndarray.empty(w.shape, rt.ctx)
+    # poison the outputs: every element must be written (beta = 0 semantics)
+    gpu_op.array_set(gy, np.nan, rt.stream)
+    gpu_op.array_set(gdx, np.nan, rt.stream)
+    gpu_op.array_set(gdw, np.nan, rt.stream)
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream) == 0
+
+    def check(got, ref, what):
+        scale = max(1.0, float(np.abs(ref).max()))
+        np.testing.assert_allclose(got, ref, rtol=1e-3, atol=1e-5 * scale, err_msg=what)
+
+    check(gy.asnumpy(), y_ref, "forward")
+    check(gdx.asnumpy(), dx_ref, "grad-data")
+    check(gdw.asnumpy(), dw_ref, "grad-filter")
+
+
+def test_conv_gradients_are_deterministic(rt):
+    """Split reductions are added in a fixed order: two runs agree bit for bit."""
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(11)
+    x = rng.normal(0, 1, (8, 64, 28, 28)).astype(np.float32)
+    w = rng.normal(0, 0.05, (64, 64, 3, 3)).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", "SAME", 1, 1)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
+    outs = []
+    for _ in range(2):
+        gdw = ndarray.empty(w.shape, rt.ctx)
+        gdx = ndarray.empty(x.shape, rt.ctx)
+        gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream)
+        gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream)
+        outs.append((gdw.asnumpy(), gdx.asnumpy()))
+    np.testing.assert_array_equal(outs[0][0], outs[1][0])
+    np.testing.assert_array_equal(outs[0][1], outs[1][1])
+
+
+def test_conv_adjoint_identities_full_size(rt):
+    """<conv(x,w), dy> = <x, dgrad(dy,w)> = <w, wgrad(x,dy)> at a full ResNet-50
+    batch-64 layer shape (too large for the CPU oracle in a unit test)."""
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(12)
+    x = rng.normal(0, 1, (64, 128, 28, 28)).astype(np.float32)
+    w = rng.normal(0, 0.03, (128, 128, 3, 3)).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", "SAME", 1, 1)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
+    gy, gdx, gdw = ndarray.empty(out_shape, rt.ctx), ndarray.empty(x.shape, rt.ctx), ndarray.empty(w.shape, rt.ctx)
+    gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream)
+    gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream)
+    gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream)
+    a = np.vdot(gy.asnumpy().astype(np.float64), dy.astype(np.float64))
+    b = np.vdot(x.astype(np.float64), gdx.asnumpy().astype(np.float64))
+    c = np.vdot(w.astype(np.float64), gdw.asnumpy().astype(np.float64))
+    assert abs(a - b) <= 1e-4 * abs(a) and abs(a - c) <= 1e-4 * abs(a)
+
+
+def test_conv_rejects_mismatched_arrays(rt, capfd):
+    from tinyflow_amd import gpu_op, ndarray
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape((2, 3, 8, 8), (4, 3, 3, 3), "NCHW", "SAME", 1, 1)
+    x = ndarray.empty((2, 3, 8, 8), rt.ctx)
+    w = ndarray.empty((4, 3, 3, 3), rt.ctx)
+    bad = ndarray.empty((2, 4, 7, 8), rt.ctx)
+    with pytest.raises(RuntimeError):
+        gpu_op.convolution_2d_forward(x, w, bad, lst, rt.cudnn, rt.stream)

@@ -1,0 +1,145 @@
+"""GPU parity of pooling, activation and batch-norm entry points against the oracle.
+
+Bit-exact: max-pool forward values, max-pool routing (which input receives each
+dy, checked with distinct dy values and with tied inputs), ReLU masks.
+fp32 within rtol 1e-3 / atol 1e-5: batch-norm reductions, softmax, mean pooling.
+"""
+import numpy as np
+import pytest
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu(a, rt):
+    from tinyflow_amd import ndarray
+    return ndarray.array(np.asarray(a, dtype=np.float32), rt.ctx)
+
+
+# (shape, mode, pad_h, pad_w, u, v, fh, fw)
+POOL_CASES = [
+    ((64, 6, 28, 28), "max", 0, 0, 2, 2, 2, 2),     # LeNet
+    ((64, 16, 10, 10), "max", 0, 0, 2, 2, 2, 2),
+    ((4, 64, 112, 112), "max", 1, 1, 2, 2, 3, 3),   # ResNet stem pool (pad 1)
+    ((4, 64, 112, 112), "max", 0, 0, 2, 2, 3, 3),   # the reference graph's pad 0 variant
+    ((8, 2048, 7, 7), "mean", 0, 0, 1, 1, 7, 7),    # global average pool
+    ((3, 5, 13, 9), "max", 1, 0, 2, 1, 3, 2),
+    ((3, 5, 13, 9), "mean", 1, 1, 2, 2, 3, 3),
+    ((2, 3, 8, 8), "max", 0, 0, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("ties", [False, True])
+def test_pooling(rt, case, ties):
+    from tinyflow_amd import gpu_op, ndarray
+    shape, mode, ph, pw, u, v, fh, fw = case
+    rng = np.random.RandomState(21)
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    if ties:  # post-ReLU style input: many exact zeros and repeated values
+        x = np.maximum(np.round(x * 2) / 2, 0).astype(np.float32)
+    out_shape, lst = gpu_op.pooling_2d_forward_get_out_shape(shape, "NCHW", mode, ph, pw, u, v, fh, fw)
+    assert out_shape[2] == O.pool_out_extent(shape[2], fh, ph, u)
+    assert out_shape[3] == O.pool_out_extent(shape[3], fw, pw, v)
+    # distinct upstream values identify where each one is routed
+    dy = (rng.permutation(int(np.prod(out_shape))).reshape(out_shape) + 1).astype(np.float32)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(out_shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    gpu_op.pooling_2d_forward(gx, gy, lst, rt.cudnn, rt.stream)
+    gpu_op.pooling_2d_backward(gx, gy, gdy, gdx, lst, rt.cudnn, rt.stream)
+    if mode == "max":
+        np.testing.assert_array_equal(gy.asnumpy(), O.max_pool_forward(x, fh, fw, ph, pw, u, v))
+        dx_ref = O.max_pool_backward(x.astype(np.float64), dy.astype(np.float64), fh, fw, ph, pw, u, v)
+        if u >= fh and v >= fw:   # disjoint windows: every dx is a single dy -> exact
+            np.testing.assert_array_equal(gdx.asnumpy(), dx_ref.astype(np.float32))
+        else:                     # overlapping windows: sums of a few dy
+            np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-6)
+        np.testing.assert_allclose(gdx.asnumpy().astype(np.float64).sum(), dy.astype(np.float64).sum(), rtol=1e-6)
+    else:
+        np.testing.assert_allclose(gy.asnumpy(), O.avg_pool_forward(x.astype(np.float64), fh, fw, ph, pw, u, v),
+                                   rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(gdx.asnumpy(),
+                                   O.avg_pool_backward(shape, dy.astype(np.float64), fh, fw, ph, pw, u, v),
+                                   rtol=1e-5)
+
+
+def test_max_pool_routing_is_first_maximum(rt):
+    """All-equal window: the gradient goes to the first position in row-major order."""
+    from tinyflow_amd import gpu_op, ndarray
+    x = np.zeros((1, 1, 4, 4), np.float32)
+    out_shape, lst = gpu_op.pooling_2d_forward_get_out_shape(x.shape, "NCHW", "max", 0, 0, 2, 2, 2, 2)
+    dy = np.arange(1, 5, dtype=np.float32).reshape(out_shape)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(out_shape, rt.ctx), ndarray.empty(x.shape, rt.ctx)
+    gpu_op.pooling_2d_forward(gx, gy, lst, rt.cudnn, rt.stream)
+    gpu_op.pooling_2d_backward(gx, gy, gdy, gdx, lst, rt.cudnn, rt.stream)
+    expect = np.zeros((4, 4), np.float32)
+    expect[0, 0], expect[0, 2], expect[2, 0], expect[2, 2] = 1, 2, 3, 4
+    np.testing.assert_array_equal(gdx.asnumpy()[0, 0], expect)
+
+
+@pytest.mark.parametrize("shape", [(64, 256, 14, 14), (3, 5, 7, 9), (128, 100), (7, 1, 33)])
+@pytest.mark.parametrize("mode", ["relu", "sigmoid", "tanh", "softmax"])
+def test_activation(rt, shape, mode):
+    from tinyflow_amd import gpu_op, ndarray
+    if mode == "softmax" and int(np.prod(shape[1:])) > 4096:
+        pytest.skip("softmax instances this large are not a use case")
+    rng = np.random.RandomState(22)
+    x = rng.normal(0, 2, shape).astype(np.float32)
+    x.flat[::5] = 0.0
+    dy = rng.normal(0, 1, shape).astype(np.float32)
+    lst = gpu_op.activation_get_cudnnlist(shape, "NCHW", mode)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    gpu_op.activation_forward(gx, gy, mode, lst, rt.cudnn, rt.stream)
+    gpu_op.activation_backward(gx, gdx, gy, gdy, mode, lst, rt.cudnn, rt.stream)
+    y_ref = O.activation_forward(x.astype(np.float64), mode)
+    dx_ref = O.activation_backward(x.astype(np.float64), y_ref, dy.astype(np.float64), mode)
+    if mode == "relu":
+        np.testing.assert_array_equal(gy.asnumpy(), y_ref.astype(np.float32))
+        np.testing.assert_array_equal(gdx.asnumpy(), dx_ref.astype(np.float32))
+        assert np.all(gdx.asnumpy().flat[::5] == 0)   # mask is x > 0
+    else:
+        np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-4, atol=1e-6)
+
+
+BN_SHAPES = [(64, 64, 28, 28), (32, 16, 7, 9), (5, 3, 4, 4), (128, 8, 6, 6), (200, 4, 3, 3), (2, 2048, 7, 7),
+             (64, 1, 100)]
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES, ids=str)
+@pytest.mark.parametrize("mode", ["pre_activation", "spatial"])
+def test_batch_norm(rt, shape, mode):
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(23)
+    x = (rng.normal(0, 1, shape) * rng.uniform(0.5, 3, (1,) + shape[1:]) + rng.normal(0, 2, (1,) + shape[1:]))
+    x = x.astype(np.float32)
+    dy = rng.normal(0, 1, shape).astype(np.float32)
+    mean_p, var_p, lst = gpu_op.bn_get_cudnnlist(shape, "NCHW", mode)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    assert gpu_op.bn_forward(gx, gy, mode, 0, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.bn_backward(gx, gdy, gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    y_ref, mean, istd = O.batch_norm_forward(x64, mode)
+    dx_ref = O.batch_norm_backward(x64, dy64, mode, mean, istd)
+    np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-3, atol=2e-5)
+    scale = max(1.0, float(np.abs(dx_ref).max()))
+    np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-3, atol=2e-5 * scale)
+    # invariants of the batch-norm gradient per statistic group:
+    #   sum(dx) = 0 and sum(dx * xhat) = istd/m * sum(dy*xhat) * (m - sum(xhat^2))
+    # (the second is 0 only in the limit eps -> 0, because sum(xhat^2) = m*var/(var+eps))
+    axes = (0,) if mode == "pre_activation" else (0,) + tuple(range(2, len(shape)))
+    dx = gdx.asnumpy().astype(np.float64)
+    xhat = (x64 - mean) * istd
+    m = np.prod([shape[a] for a in axes])
+    bound = 1e-4 * m * np.abs(dx).max() + 1e-6
+    assert np.abs(dx.sum(axis=axes)).max() <= bound
+    expect = (istd / m * (dy64 * xhat).sum(axis=axes, keepdims=True)
+              * (m - (xhat * xhat).sum(axis=axes, keepdims=True)))
+    assert np.abs((dx * xhat).sum(axis=axes, keepdims=True) - expect).max() <= 10 * bound
+    # a second backward without a forward is refused (statistics were consumed)
+    with pytest.raises(RuntimeError):
+        gpu_op.bn_backward(gx, gdy, gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream)

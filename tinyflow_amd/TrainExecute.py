@@ -1,0 +1,144 @@
+"""SGD training-step executor.
+
+Counterpart of the reference ``pycode/tinyflow/TrainExecute.py``: given a loss
+node it collects the trainable variables, differentiates, appends one ``sgd_op``
+per variable, orders everything topologically and moves each update behind the
+last reader of its parameter (``swapsgd``).  The first ``run`` infers shapes
+(which creates the C-side descriptors) and allocates one device array per node;
+later runs copy the feeds in and recompute every node in place.
+
+A step only enqueues work: nothing waits for the GPU except the read-back of a
+(1,)-shaped operand inside Add/Mul (the upstream-gradient scalar) and whatever
+the caller reads afterwards with ``asnumpy``.
+"""
+import numpy as np
+
+from . import autodiff as ad
+from . import gpu_op, ndarray
+
+
+class TrainExecutor(object):
+    """Runs forward + backward + SGD update for one loss node."""
+
+    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0)):
+        self.targetloss = targetloss
+        self.learning_rate = learning_rate
+        self.Variable_node_list = ad.get_Variable_node_list(targetloss)
+        self.Variable_node_list.reverse()
+        self.Variable_node_grad_list = ad.gradients(targetloss, self.Variable_node_list)
+        self.eval_node_list = getcomputelist(self.Variable_node_list, self.Variable_node_grad_list,
+                                             learning_rate)
+        self.ctx = ctx
+        self.topo_order = swapsgd(ad.find_topo_sort(self.eval_node_list))
+        self.node_to_shape_map = None
+        self.node_to_arr_map = {}
+        self.Variable_node_np_value = None
+        self.cudaStream = gpu_op.create_cudaStream()
+        self.cudnnHandle = gpu_op.create_cudnnHandle(self.cudaStream)
+        self.cublasHandle = gpu_op.create_cublasHandle(self.cudaStream)
+        self.isfirstrun = 0
+        self._plan = None
+
+    def infer_shape(self, feed_shapes):
+        """Shapes of every node from the shapes of the fed nodes."""
+        self.node_to_shape_map = dict(feed_shapes)
+        for node in self.topo_order:
+            if node in self.node_to_shape_map:
+                continue
+            input_shapes = [self.node_to_shape_map[i] for i in node.inputs]
+            assert None not in input_shapes
+            self.node_to_shape_map[node] = tuple(node.op.infer_shape(node, input_shapes, self.cudnnHandle))
+
+    def init_Variable(self, feed_dict):
+        """Initial values (numpy) of the trainable variables, used by the first run."""
+        self.Variable_node_np_value = feed_dict
+
+    def _alloc(self, shape):
+        arr = ndarray.empty(shape, ctx=self.ctx)
+        if isinstance(arr, int):
+            raise MemoryError("device out of memory: %d more bytes wanted" % arr)
+        return arr
+
+    def _first_run(self, feed_dict):
+        feed_dict = dict(feed_dict)
+        feed_dict.update(self.Variable_node_np_value or {})
+        self.infer_shape({node: np.shape(value) for node, value in feed_dict.items()})
+        plan = []
+        for node in self.topo_order:
+            if node in feed_dict:
+                arr = ndarray.array(feed_dict[node], ctx=self.ctx)
+                if isinstance(arr, int):
+                    raise MemoryError("device out of memory: %d more bytes wanted" % arr)
+                self.node_to_arr_map[node] = arr
+                continue
+            assert node.isw not in (1, 2), "no value fed for %s" % node.name
+            input_vals = [self.node_to_arr_map[i] for i in node.inputs]
+            if node.issgd:
+                node_val = None  # updates its parameter in place
+            else:
+                node_val = self._alloc(self.node_to_shape_map[node])
+                self.node_to_arr_map[node] = node_val
+            plan.append((node.op.compute, node, input_vals, node_val))
+        self._plan = plan
+        self.isfirstrun = 1
+
+    def run(self, feed_dict, Accuracy_node=None, convert_to_numpy_ret_vals=False):
+        """One step.  Returns [loss, variables in network order (, accuracy node)]."""
+        if self.isfirstrun == 0:
+            self._first_run(feed_dict)
+        else:
+            for node, value in feed_dict.items():
+                if node.isw == 1:
+                    continue  # variables live on the device; only data is re-fed
+                self.node_to_arr_map[node]._sync_copyfrom(value)
+        handles = (self.cudnnHandle, self.cublasHandle, self.cudaStream)
+        for compute, node, input_vals, node_val in self._plan:
+            wanted = compute(node, input_vals, node_val, *handles)
+            if wanted:
+                raise MemoryError("%s: %d bytes of device scratch could not be allocated" % (node.name, wanted))
+        result = [self.node_to_arr_map[self.targetloss]]
+        result += [self.node_to_arr_map[v] for v in reversed(self.Variable_node_list)]
+        if Accuracy_node is not None:
+            result.append(self.node_to_arr_map[Accuracy_node])
+        if convert_to_numpy_ret_vals:
+            return [r.asnumpy() for r in result]
+        return result
+
+    def value_of(self, node):
+        """Device array currently holding ``node`` (any node of the step graph)."""
+        return self.node_to_arr_map[node]
+
+
+def getcomputelist(Variable_node_list, Variable_node_grad_list, learning_rate):
+    """One in-place SGD node per variable (reference TrainExecute.py:315-324)."""
+    computelist = []
+    for var, grad in zip(Variable_node_list, Variable_node_grad_list):
+        node = ad.sgd_op(var, grad, learning_rate)
+        node.issgd = 1
+        computelist.append(node)
+    return computelist
+
+
+def swapsgd(topoorder):
+    """Move every update node to just behind the last non-update node that reads
+    its parameter, so that e.g. the grad-data convolution of a layer still sees
+    the weights the forward pass used (reference TrainExecute.py:329-349)."""
+    topoorder = list(topoorder)
+    i = 0
+    while i < len(topoorder):
+        node = topoorder[i]
+        if node.issgd == 1 and node.isw == 0:
+            node.isw = 3
+            param = node.inputs[0]
+            j = len(topoorder) - 1
+            while j > i:
+                other = topoorder[j]
+                if other.issgd != 1 and param in other.inputs:
+                    break
+                j -= 1
+            if j > i:
+                topoorder.pop(i)
+                topoorder.insert(j, node)
+                continue  # position i now holds the next node
+        i += 1
+    return topoorder

@@ -1,0 +1,414 @@
+// Batch normalisation forward (training) and backward with gamma = 1, beta = 0,
+// eps = 1e-5 and biased variance -- the only configuration the reference uses
+// (src/gpu_op.cu:4224-4458: scale/bias are rebuilt as ones/zeros on every call,
+// the scale/bias gradients cuDNN returns are discarded, there are no running
+// statistics).
+//
+// per-activation mode (what every reference model graph passes): one statistic
+//   per (c,h,w) position over the batch.  x is an [N, L] matrix, L = C*H*W; a lane
+//   owns one column, keeps its N values in registers, and the whole op is a
+//   single pass: forward reads x and writes y (8 B/element), backward reads x, dy
+//   and writes dx (12 B/element).  Lanes of a wave read 64 consecutive columns,
+//   so every access is a full 256-byte line.
+// spatial mode: one statistic per channel over (N,H,W).  Two passes: per-(channel,
+//   image-chunk) partial sums in fp64, then a normalise pass that first folds the
+//   partials of its channel in a fixed order (12 B/element forward, 20 backward).
+//
+// Saved statistics protocol (as the reference): forward allocates mean and
+// inverse-std buffers and publishes them through *mean_p / *Variance_p; backward
+// consumes and releases them.
+#include "internal.h"
+
+using namespace tf;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr float kEps = 1e-5f;
+
+// ---------------------------------------------------------------- per-activation
+
+// NREG >= N values of one column live in registers.
+template <int NREG>
+__global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__restrict__ x,
+                                                                float *__restrict__ y,
+                                                                float *__restrict__ save_mean,
+                                                                float *__restrict__ save_istd, int N, int64_t L) {
+  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (l >= L) return;
+  float v[NREG];
+#pragma unroll
+  for (int n = 0; n < NREG; ++n) v[n] = n < N ? x[(int64_t)n * L + l] : 0.f;
+  float s = 0.f;
+#pragma unroll
+  for (int n = 0; n < NREG; ++n) s += v[n];
+  const float mean = s / (float)N;
+  float q = 0.f;
+#pragma unroll
+  for (int n = 0; n < NREG; ++n) {
+    const float dlt = n < N ? v[n] - mean : 0.f;
+    q += dlt * dlt;
+  }
+  const float istd = 1.0f / sqrtf(q / (float)N + kEps);
+  save_mean[l] = mean;
+  save_istd[l] = istd;
+#pragma unroll
+  for (int n = 0; n < NREG; ++n)
+    if (n < N) y[(int64_t)n * L + l] = (v[n] - mean) * istd;
+}
+
+// any N: three sweeps over the column (the second and third hit the cache)
+__global__ __launch_bounds__(kThreads) void bn_pa_forward_stream_kernel(const float *__restrict__ x,
+                                                                       float *__restrict__ y,
+                                                                       float *__restrict__ save_mean,
+                                                                       float *__restrict__ save_istd, int N,
+                                                                       int64_t L) {
+  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (l >= L) return;
+  float s = 0.f;
+  for (int n = 0; n < N; ++n) s += x[(int64_t)n * L + l];
+  const float mean = s / (float)N;
+  float q = 0.f;
+  for (int n = 0; n < N; ++n) {
+    const float dlt = x[(int64_t)n * L + l] - mean;
+    q += dlt * dlt;
+  }
+  const float istd = 1.0f / sqrtf(q / (float)N + kEps);
+  save_mean[l] = mean;
+  save_istd[l] = istd;
+  for (int n = 0; n < N; ++n) y[(int64_t)n * L + l] = (x[(int64_t)n * L + l] - mean) * istd;
+}
+
+// dx = istd/N * (N*dy - sum(dy) - xhat * sum(dy*xhat))
+template <int NREG>
+__global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *__restrict__ x,
+                                                                 const float *__restrict__ dy,
+                                                                 float *__restrict__ dx,
+                                                                 const float *__restrict__ save_mean,
+                                                                 const float *__restrict__ save_istd, int N,
+                                                                 int64_t L) {
+  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (l >= L) return;
+  const float mean = save_mean[l], istd = save_istd[l];
+  float xh[NREG], g[NREG];
+#pragma unroll
+  for (int n = 0; n < NREG; ++n) {
+    xh[n] = n < N ? x[(int64_t)n * L + l] : mean;
+    g[n] = n < N ? dy[(int64_t)n * L + l] : 0.f;
+  }
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int n = 0; n < NREG; ++n) {
+    xh[n] = (xh[n] - mean) * istd;
+    s1 += g[n];
+    s2 += g[n] * xh[n];
+  }
+  const float m = (float)N;
+  const float scale = istd / m;
+#pragma unroll
+  for (int n = 0; n < NREG; ++n)
+    if (n < N) dx[(int64_t)n * L + l] = scale * (m * g[n] - s1 - xh[n] * s2);
+}
+
+__global__ __launch_bounds__(kThreads) void bn_pa_backward_stream_kernel(const float *__restrict__ x,
+                                                                        const float *__restrict__ dy,
+                                                                        float *__restrict__ dx,
+                                                                        const float *__restrict__ save_mean,
+                                                                        const float *__restrict__ save_istd,
+                                                                        int N, int64_t L) {
+  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (l >= L) return;
+  const float mean = save_mean[l], istd = save_istd[l];
+  float s1 = 0.f, s2 = 0.f;
+  for (int n = 0; n < N; ++n) {
+    const float g = dy[(int64_t)n * L + l];
+    s1 += g;
+    s2 += g * ((x[(int64_t)n * L + l] - mean) * istd);
+  }
+  const float m = (float)N;
+  const float scale = istd / m;
+  for (int n = 0; n < N; ++n) {
+    const float xh = (x[(int64_t)n * L + l] - mean) * istd;
+    dx[(int64_t)n * L + l] = scale * (m * dy[(int64_t)n * L + l] - s1 - xh * s2);
+  }
+}
+
+// ------------------------------------------------------------------------ spatial
+
+__device__ inline double wave_sum_d(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+// Sum of a pair over the 256 lanes of a block, valid in thread 0.
+__device__ inline void block_sum2(double &a, double &b, double (*smem)[2]) {
+  a = wave_sum_d(a);
+  b = wave_sum_d(b);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    smem[wave][0] = a;
+    smem[wave][1] = b;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    a = (smem[0][0] + smem[1][0]) + (smem[2][0] + smem[3][0]);
+    b = (smem[0][1] + smem[1][1]) + (smem[2][1] + smem[3][1]);
+  }
+}
+
+// x viewed as [N, C, HW]; block (c, chunk) sums images [chunk*ipc, ...) of channel c.
+// FWD: partial = (sum x, sum x^2); BWD: partial = (sum dy, sum dy*xhat)
+template <bool BWD>
+__global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__restrict__ x,
+                                                                const float *__restrict__ dy,
+                                                                const float *__restrict__ save_mean,
+                                                                const float *__restrict__ save_istd,
+                                                                double *__restrict__ partial, int N, int C,
+                                                                int HW, int images_per_chunk) {
+  __shared__ double smem[4][2];
+  const int c = blockIdx.x;
+  const int n0 = blockIdx.y * images_per_chunk;
+  int n1 = n0 + images_per_chunk;
+  if (n1 > N) n1 = N;
+  const float mean = BWD ? save_mean[c] : 0.f, istd = BWD ? save_istd[c] : 0.f;
+  float a0 = 0.f, b0 = 0.f;
+  double a = 0.0, b = 0.0;
+  for (int n = n0; n < n1; ++n) {
+    const int64_t row = ((int64_t)n * C + c) * HW;
+    a0 = 0.f;
+    b0 = 0.f;
+    for (int i = threadIdx.x; i < HW; i += kThreads) {
+      const float xv = x[row + i];
+      if (BWD) {
+        const float g = dy[row + i];
+        a0 += g;
+        b0 += g * ((xv - mean) * istd);
+      } else {
+        a0 += xv;
+        b0 += xv * xv;
+      }
+    }
+    a += (double)a0;  // per-image fp32 partials, accumulated across images in fp64
+    b += (double)b0;
+  }
+  block_sum2(a, b, smem);
+  if (threadIdx.x == 0) {
+    partial[((int64_t)blockIdx.y * C + c) * 2 + 0] = a;
+    partial[((int64_t)blockIdx.y * C + c) * 2 + 1] = b;
+  }
+}
+
+// one block per (n, c) row of HW elements; folds the channel's partials first
+__global__ __launch_bounds__(kThreads) void bn_sp_forward_apply_kernel(const float *__restrict__ x,
+                                                                      float *__restrict__ y,
+                                                                      const double *__restrict__ partial,
+                                                                      float *__restrict__ save_mean,
+                                                                      float *__restrict__ save_istd, int N,
+                                                                      int C, int HW, int chunks) {
+  const int c = blockIdx.x % C;
+  double s = 0.0, q = 0.0;
+  for (int k = 0; k < chunks; ++k) {
+    s += partial[((int64_t)k * C + c) * 2 + 0];
+    q += partial[((int64_t)k * C + c) * 2 + 1];
+  }
+  const double m = (double)N * (double)HW;
+  const double mean_d = s / m;
+  double var = q / m - mean_d * mean_d;
+  if (var < 0.0) var = 0.0;
+  const float mean = (float)mean_d;
+  const float istd = (float)(1.0 / sqrt(var + (double)kEps));
+  if (blockIdx.x < C && threadIdx.x == 0) {  // rows of image 0 publish the statistics
+    save_mean[c] = mean;
+    save_istd[c] = istd;
+  }
+  const int64_t row = (int64_t)blockIdx.x * HW;
+  for (int i = threadIdx.x; i < HW; i += kThreads) y[row + i] = (x[row + i] - mean) * istd;
+}
+
+__global__ __launch_bounds__(kThreads) void bn_sp_backward_apply_kernel(const float *__restrict__ x,
+                                                                       const float *__restrict__ dy,
+                                                                       float *__restrict__ dx,
+                                                                       const double *__restrict__ partial,
+                                                                       const float *__restrict__ save_mean,
+                                                                       const float *__restrict__ save_istd,
+                                                                       int N, int C, int HW, int chunks) {
+  const int c = blockIdx.x % C;
+  double s1d = 0.0, s2d = 0.0;
+  for (int k = 0; k < chunks; ++k) {
+    s1d += partial[((int64_t)k * C + c) * 2 + 0];
+    s2d += partial[((int64_t)k * C + c) * 2 + 1];
+  }
+  const float mean = save_mean[c], istd = save_istd[c];
+  const float m = (float)((double)N * (double)HW);
+  const float s1 = (float)s1d, s2 = (float)s2d;
+  const float scale = istd / m;
+  const int64_t row = (int64_t)blockIdx.x * HW;
+  for (int i = threadIdx.x; i < HW; i += kThreads) {
+    const float xh = (x[row + i] - mean) * istd;
+    dx[row + i] = scale * (m * dy[row + i] - s1 - xh * s2);
+  }
+}
+
+int sp_chunks(int N, int C) {
+  // about four workgroups per CU in the partial pass
+  int chunks = cdiv((int64_t)num_cus() * 4, C);
+  if (chunks > N) chunks = N;
+  return chunks < 1 ? 1 : chunks;
+}
+
+int check_bn_arrays(const BNDesc *d, const DLArray *a, const DLArray *b) {
+  TF_REQUIRE(on_gpu(a) && on_gpu(b), "arrays must live on the GPU");
+  const int64_t n = (int64_t)d->N * d->C * d->HW;
+  TF_REQUIRE(numel(a) == n && numel(b) == n, "arrays do not match the descriptor");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int DLGpuBatchNormalizationGetCudnnlist(const int *input_shapes, int sizeofshape, int dataformat,
+                                                   int batchNormMode, void **mean_p, void **Variance_p,
+                                                   void ***list) {
+  (void)mean_p;
+  (void)Variance_p;
+  TF_REQUIRE(input_shapes && list, "null argument");
+  TF_REQUIRE(sizeofshape >= 2 && sizeofshape <= 5, "rank %d not supported", sizeofshape);
+  TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
+  TF_REQUIRE(batchNormMode == 0 || batchNormMode == 1, "unknown batch-norm mode %d", batchNormMode);
+  BNDesc *d = new BNDesc();
+  d->magic = kMagicBN;
+  d->mode = batchNormMode;
+  d->N = input_shapes[0];
+  d->C = input_shapes[1];
+  int64_t hw = 1;
+  for (int i = 2; i < sizeofshape; ++i) hw *= input_shapes[i];
+  TF_REQUIRE(hw <= INT32_MAX, "spatial extent too large");
+  d->HW = (int)hw;
+  d->stat_count = batchNormMode == 0 ? (int64_t)d->C * d->HW : d->C;
+  d->saved_mean = d->saved_istd = nullptr;
+  void **slots = (void **)malloc(sizeof(void *) * 3);
+  slots[0] = slots[1] = slots[2] = d;
+  *list = slots;
+  return 0;
+}
+
+extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArrayHandle output,
+                                              int batchNormMode, int n, void **mean_p, void **Variance_p,
+                                              void ***list, void **handle, int *memorytoSaving,
+                                              void **stream) {
+  (void)handle;
+  (void)n;  // would weight running statistics, which the reference never keeps
+  BNDesc *d = desc_from_list<BNDesc>(list, kMagicBN);
+  TF_REQUIRE(d, "descriptor list was not created by DLGpuBatchNormalizationGetCudnnlist");
+  TF_REQUIRE(d->mode == batchNormMode, "mode differs from the descriptor");
+  TF_REQUIRE(mean_p && Variance_p, "null statistics cell");
+  if (check_bn_arrays(d, input, output) != 0) return -1;
+  hipStream_t s = stream_of(stream);
+  const size_t stat_bytes = (size_t)d->stat_count * sizeof(float);
+  if (d->saved_mean) {  // a forward whose backward never ran: recycle its statistics
+    device_free(d->saved_mean);
+    device_free(d->saved_istd);
+    d->saved_mean = d->saved_istd = nullptr;
+  }
+  float *mean = (float *)device_alloc(stat_bytes);
+  float *istd = mean ? (float *)device_alloc(stat_bytes) : nullptr;
+  if (!mean || !istd) {
+    if (mean) device_free(mean);
+    if (memorytoSaving) *memorytoSaving = (int)stat_bytes;
+    return 0;
+  }
+  *mean_p = d->saved_mean = mean;
+  *Variance_p = d->saved_istd = istd;
+  const float *x = (const float *)input->data;
+  float *y = (float *)output->data;
+  if (numel(input) == 0) return 0;
+  if (d->mode == 0) {
+    const int64_t L = d->stat_count;
+    const dim3 grid(cdiv(L, kThreads)), block(kThreads);
+    if (d->N <= 32)
+      hipLaunchKernelGGL(bn_pa_forward_kernel<32>, grid, block, 0, s, x, y, mean, istd, d->N, L);
+    else if (d->N <= 64)
+      hipLaunchKernelGGL(bn_pa_forward_kernel<64>, grid, block, 0, s, x, y, mean, istd, d->N, L);
+    else if (d->N <= 128)
+      hipLaunchKernelGGL(bn_pa_forward_kernel<128>, grid, block, 0, s, x, y, mean, istd, d->N, L);
+    else
+      hipLaunchKernelGGL(bn_pa_forward_stream_kernel, grid, block, 0, s, x, y, mean, istd, d->N, L);
+  } else {
+    const int chunks = sp_chunks(d->N, d->C);
+    const int ipc = cdiv(d->N, chunks);
+    const int real_chunks = cdiv(d->N, ipc);
+    const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double);
+    double *partial = (double *)device_alloc(pbytes);
+    if (!partial) {
+      device_free(mean);
+      device_free(istd);
+      *mean_p = d->saved_mean = nullptr;
+      *Variance_p = d->saved_istd = nullptr;
+      if (memorytoSaving) *memorytoSaving = (int)pbytes;
+      return 0;
+    }
+    hipLaunchKernelGGL(bn_sp_partial_kernel<false>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x,
+                       (const float *)nullptr, (const float *)nullptr, (const float *)nullptr, partial, d->N,
+                       d->C, d->HW, ipc);
+    hipLaunchKernelGGL(bn_sp_forward_apply_kernel, dim3((unsigned)d->N * d->C), dim3(kThreads), 0, s, x, y,
+                       partial, mean, istd, d->N, d->C, d->HW, real_chunks);
+    device_free(partial);
+  }
+  return finish(s, "DLGpuBatchNormalizationForward");
+}
+
+extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const DLArrayHandle doutput,
+                                               DLArrayHandle dinput, int batchNormMode, void **mean_p,
+                                               void **Variance_p, void ***list, void **handle,
+                                               int *memorytoSaving, void **stream) {
+  (void)handle;
+  BNDesc *d = desc_from_list<BNDesc>(list, kMagicBN);
+  TF_REQUIRE(d, "descriptor list was not created by DLGpuBatchNormalizationGetCudnnlist");
+  TF_REQUIRE(d->mode == batchNormMode, "mode differs from the descriptor");
+  // the cells start out pointing at host integers, so "non-null" proves nothing:
+  // they must hold exactly what the last forward published
+  TF_REQUIRE(mean_p && Variance_p && d->saved_mean && *mean_p == d->saved_mean &&
+                 *Variance_p == d->saved_istd,
+             "no saved statistics: backward needs the forward pass of the same step");
+  if (check_bn_arrays(d, input, doutput) != 0) return -1;
+  TF_REQUIRE(on_gpu(dinput) && numel(dinput) == numel(input), "dinput must have the input's shape");
+  hipStream_t s = stream_of(stream);
+  const float *x = (const float *)input->data, *dy = (const float *)doutput->data;
+  float *dx = (float *)dinput->data;
+  const float *mean = (const float *)*mean_p, *istd = (const float *)*Variance_p;
+  if (numel(input) != 0) {
+    if (d->mode == 0) {
+      const int64_t L = d->stat_count;
+      const dim3 grid(cdiv(L, kThreads)), block(kThreads);
+      if (d->N <= 32)
+        hipLaunchKernelGGL(bn_pa_backward_kernel<32>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+      else if (d->N <= 64)
+        hipLaunchKernelGGL(bn_pa_backward_kernel<64>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+      else if (d->N <= 128)
+        hipLaunchKernelGGL(bn_pa_backward_kernel<128>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+      else
+        hipLaunchKernelGGL(bn_pa_backward_stream_kernel, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+    } else {
+      const int chunks = sp_chunks(d->N, d->C);
+      const int ipc = cdiv(d->N, chunks);
+      const int real_chunks = cdiv(d->N, ipc);
+      const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double);
+      double *partial = (double *)device_alloc(pbytes);
+      if (!partial) {
+        if (memorytoSaving) *memorytoSaving = (int)pbytes;
+        return 0;  // statistics stay published so the call can be repeated
+      }
+      hipLaunchKernelGGL(bn_sp_partial_kernel<true>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x, dy,
+                         mean, istd, partial, d->N, d->C, d->HW, ipc);
+      hipLaunchKernelGGL(bn_sp_backward_apply_kernel, dim3((unsigned)d->N * d->C), dim3(kThreads), 0, s, x,
+                         dy, dx, partial, mean, istd, d->N, d->C, d->HW, real_chunks);
+      device_free(partial);
+    }
+  }
+  // the saved statistics are consumed (stream-ordered release)
+  device_free(d->saved_mean);
+  device_free(d->saved_istd);
+  *mean_p = d->saved_mean = nullptr;
+  *Variance_p = d->saved_istd = nullptr;
+  return finish(s, "DLGpuBatchNormalizationBackward");
+}

@@ -43,7 +43,8 @@ __device__ inline float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
 struct FastDiv {
   uint32_t d, mul, shift;
   FastDiv() : d(1), mul(0), shift(0) {}
-  explicit FastDiv(uint32_t div) : d(div) {
+  explicit FastDiv(uint32_t div) : d(div ? div : 1) {
+    div = d;
     uint32_t l = 0;
     while ((1ull << l) < div) ++l;
     shift = l;

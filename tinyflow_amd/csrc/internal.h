@@ -111,6 +111,8 @@ struct BNDesc {
   int mode;            // 0 per-activation, 1 spatial
   int N, C, HW;        // x viewed as [N, C, HW]
   int64_t stat_count;  // C*HW (per-activation) or C (spatial)
+  // statistics published by the last forward and not yet consumed by a backward
+  float *saved_mean, *saved_istd;
 };
 
 struct ReduceDesc {

@@ -1,0 +1,208 @@
+// 2-D pooling forward/backward (max, and mean with padding counted).
+//
+// Replaces cudnnPoolingForward / cudnnPoolingBackward and the descriptor
+// builder (src/gpu_op.cu:2839-3024).  NCHW; lanes run along the innermost (w / q)
+// index so loads and stores coalesce.
+//
+// Max-pool backward is a gather: one lane per INPUT pixel looks at the (few)
+// windows that cover it and takes dy from those whose maximum it is.  Among
+// equal maxima the first one in row-major window order wins, so the result is
+// deterministic and needs no atomics even when windows overlap (3x3 stride 2).
+#include "internal.h"
+
+using namespace tf;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct PoolParams {
+  int C, H, W, P, Q;
+  int pad_h, pad_w, u, v, fh, fw;
+};
+
+template <bool MAX>
+__global__ __launch_bounds__(kThreads) void pool_forward_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                               PoolParams pp, int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int q = (int)(i % pp.Q);
+    const int64_t t = i / pp.Q;
+    const int p = (int)(t % pp.P);
+    const int64_t nc = t / pp.P;
+    const float *plane = x + nc * pp.H * pp.W;
+    const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+    float acc = MAX ? -INFINITY : 0.f;
+    for (int r = 0; r < pp.fh; ++r) {
+      const int h = h0 + r;
+      if ((unsigned)h >= (unsigned)pp.H) continue;
+      for (int s = 0; s < pp.fw; ++s) {
+        const int w = w0 + s;
+        if ((unsigned)w >= (unsigned)pp.W) continue;
+        const float val = plane[h * pp.W + w];
+        if (MAX) acc = val > acc ? val : acc;
+        else acc += val;
+      }
+    }
+    y[i] = MAX ? acc : acc / (float)(pp.fh * pp.fw);
+  }
+}
+
+__device__ inline int ceil_div_floor0(int a, int b) {  // ceil(a / b) clamped at 0, b > 0
+  return a <= 0 ? 0 : (a + b - 1) / b;
+}
+
+template <bool MAX>
+__global__ __launch_bounds__(kThreads) void pool_backward_kernel(const float *__restrict__ x,
+                                                                const float *__restrict__ y,
+                                                                const float *__restrict__ dy,
+                                                                float *__restrict__ dx, PoolParams pp,
+                                                                int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int w = (int)(i % pp.W);
+    const int64_t t = i / pp.W;
+    const int h = (int)(t % pp.H);
+    const int64_t nc = t / pp.H;
+    // windows (p, q) with p*u - pad <= h <= p*u - pad + fh - 1
+    const int p_lo = ceil_div_floor0(h + pp.pad_h - pp.fh + 1, pp.u);
+    int p_hi = (h + pp.pad_h) / pp.u;
+    if (p_hi > pp.P - 1) p_hi = pp.P - 1;
+    const int q_lo = ceil_div_floor0(w + pp.pad_w - pp.fw + 1, pp.v);
+    int q_hi = (w + pp.pad_w) / pp.v;
+    if (q_hi > pp.Q - 1) q_hi = pp.Q - 1;
+    const float *xp = x + nc * pp.H * pp.W;
+    const float *yp = y + nc * pp.P * pp.Q;
+    const float *dyp = dy + nc * pp.P * pp.Q;
+    const float mine = MAX ? xp[h * pp.W + w] : 0.f;
+    float acc = 0.f;
+    for (int p = p_lo; p <= p_hi; ++p)
+      for (int q = q_lo; q <= q_hi; ++q) {
+        if (!MAX) {
+          acc += dyp[p * pp.Q + q];
+          continue;
+        }
+        if (mine != yp[p * pp.Q + q]) continue;
+        // this pixel holds the window's maximum; it receives dy unless an
+        // earlier position (row-major) of the same window holds it too
+        const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+        bool first = true;
+        for (int r = 0; r < pp.fh && first; ++r) {
+          const int hh = h0 + r;
+          if (hh > h) break;
+          if (hh < 0) continue;
+          for (int s = 0; s < pp.fw; ++s) {
+            const int ww = w0 + s;
+            if (hh == h && ww >= w) break;
+            if ((unsigned)ww >= (unsigned)pp.W) continue;
+            if (xp[hh * pp.W + ww] == mine) {
+              first = false;
+              break;
+            }
+          }
+        }
+        if (first) acc += dyp[p * pp.Q + q];
+      }
+    dx[i] = MAX ? acc : acc / (float)(pp.fh * pp.fw);
+  }
+}
+
+int grid_for(int64_t n) {
+  int64_t blocks = (n + kThreads - 1) / kThreads;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  return blocks < 1 ? 1 : (int)blocks;
+}
+
+PoolParams params_of(const PoolDesc *d) {
+  return PoolParams{d->C, d->H, d->W, d->P, d->Q, d->pad_h, d->pad_w, d->u, d->v, d->fh, d->fw};
+}
+
+bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
+  return a->ndim == 4 && a->shape[0] == d0 && a->shape[1] == d1 && a->shape[2] == d2 && a->shape[3] == d3;
+}
+
+}  // namespace
+
+extern "C" int DLGpuPooling2DForwardGetOutShape(const int *input_shapes, int *output_shapes, int dataformat,
+                                                int poolingMode, const int padding_h, const int padding_w,
+                                                const int u, const int v, const int filter_h,
+                                                const int filter_w, void ***list) {
+  TF_REQUIRE(input_shapes && output_shapes && list, "null argument");
+  TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
+  TF_REQUIRE(poolingMode == 0 || poolingMode == 1, "unknown pooling mode %d", poolingMode);
+  TF_REQUIRE(u >= 1 && v >= 1 && filter_h >= 1 && filter_w >= 1 && padding_h >= 0 && padding_w >= 0,
+             "bad window geometry");
+  PoolDesc *d = new PoolDesc();
+  d->magic = kMagicPool;
+  d->N = input_shapes[0];
+  d->C = input_shapes[1];
+  d->H = input_shapes[2];
+  d->W = input_shapes[3];
+  d->mode = poolingMode;
+  d->pad_h = padding_h;
+  d->pad_w = padding_w;
+  d->u = u;
+  d->v = v;
+  d->fh = filter_h;
+  d->fw = filter_w;
+  TF_REQUIRE(d->H + 2 * padding_h >= filter_h && d->W + 2 * padding_w >= filter_w,
+             "window larger than padded input");
+  d->P = 1 + (d->H + 2 * padding_h - filter_h) / u;
+  d->Q = 1 + (d->W + 2 * padding_w - filter_w) / v;
+  output_shapes[0] = d->N;
+  output_shapes[1] = d->C;
+  output_shapes[2] = d->P;
+  output_shapes[3] = d->Q;
+  void **slots = (void **)malloc(sizeof(void *) * 3);
+  slots[0] = slots[1] = slots[2] = d;
+  *list = slots;
+  return 0;
+}
+
+extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle output, void ***list,
+                                     void **handle, void **stream) {
+  (void)handle;
+  PoolDesc *d = desc_from_list<PoolDesc>(list, kMagicPool);
+  TF_REQUIRE(d, "descriptor list was not created by DLGpuPooling2DForwardGetOutShape");
+  TF_REQUIRE(on_gpu(input) && on_gpu(output), "arrays must live on the GPU");
+  TF_REQUIRE(shape_is(input, d->N, d->C, d->H, d->W) && shape_is(output, d->N, d->C, d->P, d->Q),
+             "arrays do not match the descriptor");
+  hipStream_t s = stream_of(stream);
+  const int64_t total = numel(output);
+  if (total == 0) return 0;
+  const PoolParams pp = params_of(d);
+  if (d->mode == 0)
+    hipLaunchKernelGGL(pool_forward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s,
+                       (const float *)input->data, (float *)output->data, pp, total);
+  else
+    hipLaunchKernelGGL(pool_forward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
+                       (const float *)input->data, (float *)output->data, pp, total);
+  return finish(s, "DLGpuPooling2DForward");
+}
+
+extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHandle output,
+                                      const DLArrayHandle doutput, DLArrayHandle dinput, void ***list,
+                                      void **handle, void **stream) {
+  (void)handle;
+  PoolDesc *d = desc_from_list<PoolDesc>(list, kMagicPool);
+  TF_REQUIRE(d, "descriptor list was not created by DLGpuPooling2DForwardGetOutShape");
+  TF_REQUIRE(on_gpu(input) && on_gpu(output) && on_gpu(doutput) && on_gpu(dinput),
+             "arrays must live on the GPU");
+  TF_REQUIRE(shape_is(input, d->N, d->C, d->H, d->W) && shape_is(dinput, d->N, d->C, d->H, d->W) &&
+                 shape_is(output, d->N, d->C, d->P, d->Q) && shape_is(doutput, d->N, d->C, d->P, d->Q),
+             "arrays do not match the descriptor");
+  hipStream_t s = stream_of(stream);
+  const int64_t total = numel(dinput);
+  if (total == 0) return 0;
+  const PoolParams pp = params_of(d);
+  if (d->mode == 0)
+    hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s,
+                       (const float *)input->data, (const float *)output->data, (const float *)doutput->data,
+                       (float *)dinput->data, pp, total);
+  else
+    hipLaunchKernelGGL(pool_backward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
+                       (const float *)input->data, (const float *)output->data, (const float *)doutput->data,
+                       (float *)dinput->data, pp, total);
+  return finish(s, "DLGpuPooling2DBackward");
+}
