@@ -1,0 +1,250 @@
+"""Headline benchmark: train imgs/sec of one full training step (forward +
+backward + SGD update) of ResNet-50, batch 64, fp32, on one MI355X, synthetic data.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  Next to the throughput it carries
+  "roofline":     achieved vs peak for the kernel variant that takes the most GPU
+                  time in the step (an MFMA implicit-GEMM convolution), measured
+                  with HIP events recorded on the compute stream around every
+                  convolution launch of the timed steps;
+  "cpu_baseline": the CPU oracle (numpy restatement of the same step) timed on
+                  this machine's host cores on a bounded sample (a smaller batch),
+                  scaled linearly to images/sec.
+Everything here runs on one GPU; --gpus N with N > 1 is refused.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+
+class Hip(object):
+    """The few HIP runtime calls the benchmark needs for event timing."""
+
+    def __init__(self):
+        self.lib = ctypes.CDLL("libamdhip64.so")
+        self.lib.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.lib.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.lib.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.lib.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError("%s failed with hipError %d" % (what, rc))
+
+    def event(self):
+        ev = ctypes.c_void_p()
+        self.check(self.lib.hipEventCreate(ctypes.byref(ev)), "hipEventCreate")
+        return ev
+
+    def record(self, ev, stream):
+        self.check(self.lib.hipEventRecord(ev, stream), "hipEventRecord")
+
+    def elapsed_ms(self, e0, e1):
+        ms = ctypes.c_float()
+        self.check(self.lib.hipEventElapsedTime(ctypes.byref(ms), e0, e1), "hipEventElapsedTime")
+        return ms.value
+
+    def sync(self):
+        self.check(self.lib.hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+def stream_handle(stream_cell):
+    """hipStream_t stored in the cell that DLGpuCreatecudaStream filled."""
+    return ctypes.cast(stream_cell, ctypes.POINTER(ctypes.c_void_p))[0]
+
+
+class ConvTimer(object):
+    """Records a HIP event pair on the compute stream around every convolution
+    launch and attributes the time to the kernel variant the library reports."""
+
+    def __init__(self, hip, gpu_op, lib):
+        self.hip, self.gpu_op, self.lib = hip, gpu_op, lib
+        self.pairs = []     # (variant, flops, e0, e1)
+        self.pool = []
+        self.enabled = False
+        self._describe_cache = {}
+        self._orig = {}
+        for which, name in ((0, "convolution_2d_forward"), (1, "convolution_backward_data"),
+                            (2, "convolution_backward_filter")):
+            self._orig[name] = getattr(gpu_op, name)
+            setattr(gpu_op, name, self._wrap(which, self._orig[name]))
+
+    def _describe(self, cudnnlist, which):
+        key = (ctypes.addressof(cudnnlist.contents), which)
+        hit = self._describe_cache.get(key)
+        if hit is None:
+            buf = ctypes.create_string_buffer(96)
+            flops = ctypes.c_double()
+            rc = self.lib.DLGpuConvolutionDescribeKernel(cudnnlist, which, buf, 96, ctypes.byref(flops))
+            if rc != 0:
+                raise RuntimeError("DLGpuConvolutionDescribeKernel failed")
+            hit = (buf.value.decode(), flops.value)
+            self._describe_cache[key] = hit
+        return hit
+
+    def _event(self):
+        return self.pool.pop() if self.pool else self.hip.event()
+
+    def _wrap(self, which, fn):
+        def timed(*args):
+            if not self.enabled:
+                return fn(*args)
+            # (x, w|dy, y|w, out, cudnnlist, handle, stream) / forward: (x, w, y, cudnnlist, handle, stream)
+            cudnnlist, stream = args[-3], args[-1]
+            variant, flops = self._describe(cudnnlist, which)
+            s = stream_handle(stream)
+            e0, e1 = self._event(), self._event()
+            self.hip.record(e0, s)
+            ret = fn(*args)
+            self.hip.record(e1, s)
+            self.pairs.append((variant, flops, e0, e1))
+            return ret
+        return timed
+
+    def collect(self):
+        """{variant: [launches, total_ms, total_flops]}; call after a device sync."""
+        stats = {}
+        for variant, flops, e0, e1 in self.pairs:
+            ms = self.hip.elapsed_ms(e0, e1)
+            st = stats.setdefault(variant, [0, 0.0, 0.0])
+            st[0] += 1
+            st[1] += ms
+            st[2] += flops
+            self.pool += [e0, e1]
+        self.pairs = []
+        return stats
+
+
+def cpu_baseline(bn_mode, sample_batch, image, repeats):
+    """The oracle's ResNet-50 step on the host cores, on a reduced batch."""
+    from oracle import models as OM
+    from tinyflow_amd import models
+    model, X, y = models.build("resnet50", batch=sample_batch, image=image, bn_mode=bn_mode)
+    params = {v.name: val for v, val in model.variables.items()}
+    net = OM.network("resnet50", bn_mode=bn_mode, image=image)
+    times = []
+    for _ in range(repeats + 1):
+        t0 = time.perf_counter()
+        OM.train_step(net, params, X, y, 0.01)
+        times.append(time.perf_counter() - t0)
+    best = float(np.median(times[1:]))  # first call warms BLAS and the allocator
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = len(os.sched_getaffinity(0))
+    return {
+        "value": sample_batch / best, "unit": "imgs/sec", "cores": threads, "kind": "port",
+        "sample": "oracle numpy fp32 ResNet-50 step (fwd+bwd+SGD, bn_mode=%s) at batch %d, image %d; "
+                  "median of %d steps after 1 warm-up, %.2f s per step; images/sec = batch / time "
+                  "(os.cpu_count()=%d, affinity=%d)"
+                  % (bn_mode, sample_batch, image, repeats, best, os.cpu_count(), len(os.sched_getaffinity(0))),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--bn-mode", default="pre_activation", choices=["pre_activation", "spatial"],
+                    help="pre_activation is what every model graph of the reference passes")
+    ap.add_argument("--config", default="resnet50", choices=["resnet50", "vgg16", "lenet5", "mlp", "resnet152"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--no-kernel-events", action="store_true",
+                    help="do not record per-convolution HIP events in the timed region")
+    ap.add_argument("--breakdown", action="store_true", help="print per-variant conv times to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)\n"
+                         % args.gpus)
+        sys.exit(2)
+
+    from tinyflow_amd import gpu_op, models
+    from tinyflow_amd._base import _LIB
+    from tinyflow_amd.TrainExecute import TrainExecutor
+
+    hip = Hip()
+    timer = ConvTimer(hip, gpu_op, _LIB)
+    kw = {"batch": args.batch}
+    if args.config.startswith("resnet"):
+        kw["bn_mode"] = args.bn_mode
+    model, X, y = models.build(args.config, **kw)
+    ex = TrainExecutor(model.loss, 0.01)
+    ex.init_Variable(dict(model.variables))
+    feed = {model.X: X, model.y_: y}
+
+    for _ in range(max(args.warmup, 1)):
+        loss = ex.run(feed)[0]
+    hip.sync()
+
+    timer.enabled = not args.no_kernel_events
+    e_start, e_end = hip.event(), hip.event()
+    s = stream_handle(ex.cudaStream)
+    hip.sync()
+    t0 = time.perf_counter()
+    hip.record(e_start, s)
+    for _ in range(args.steps):
+        loss = ex.run(feed)[0]
+    hip.record(e_end, s)
+    hip.sync()
+    wall = time.perf_counter() - t0
+    timer.enabled = False
+    gpu_ms = hip.elapsed_ms(e_start, e_end)
+    loss_val = float(loss.asnumpy()[0])
+
+    ms_per_step = wall * 1e3 / args.steps
+    imgs_per_sec = args.batch * args.steps / wall
+
+    roofline = None
+    stats = timer.collect()
+    if stats:
+        top = max(stats.items(), key=lambda kv: kv[1][1])
+        name, (launches, total_ms, total_flops) = top
+        achieved = total_flops / (total_ms * 1e-3) / 1e12
+        roofline = {
+            "bound": "mfma", "kernel": name, "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+            "launches": launches, "avg_launch_ms": total_ms / launches,
+            "share_of_step": total_ms / args.steps / (gpu_ms / args.steps),
+        }
+        if args.breakdown:
+            conv_ms = sum(v[1] for v in stats.values()) / args.steps
+            sys.stderr.write("GPU ms/step (events): %.3f, conv kernels: %.3f\n" % (gpu_ms / args.steps, conv_ms))
+            for k, (n, ms, fl) in sorted(stats.items(), key=lambda kv: -kv[1][1]):
+                sys.stderr.write("  %-34s launches/step %5.1f  ms/step %8.3f  TFLOP/s %7.2f\n"
+                                 % (k, n / args.steps, ms / args.steps, fl / (ms * 1e-3) / 1e12))
+
+    result = {
+        "metric": "train imgs/sec ResNet-50 b64 fp32 fwd+bwd; bwd kernel % of HBM/MFMA peak",
+        "value": imgs_per_sec, "unit": "imgs/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s batch %d fp32 3x224x224, fwd+bwd+SGD(lr 0.01), BN mode %s, "
+                               "softmax-xent over %d random one-hot classes, He-normal weights"
+                               % (args.config, args.batch, args.bn_mode, model.n_class)},
+        "gpu_ms_per_step": gpu_ms / args.steps, "loss": loss_val,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.bn_mode, args.cpu_batch, 224, 2)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -120,9 +120,9 @@ int DLGpuMatrixElementwiseMultiply(const DLArrayHandle matA, const DLArrayHandle
 int DLGpuMatrixMultiplyByConst(const DLArrayHandle input, float val,
                                DLArrayHandle output, void **stream);
 
-/* out = max(in, 0) / out = in > 0 ? grad : 0.  Neither takes a stream; both
- * are ordered after all previously enqueued work and complete before
- * returning.  ref: c_runtime_api.h:162-172, gpu_op.cu:221-235, 1201-1233 */
+/* out = max(in, 0) / out = in > 0 ? grad : 0.  Neither takes a stream; both run
+ * on the default stream, ordered after all work already enqueued on the streams
+ * created by DLGpuCreatecudaStream and before any work enqueued there later.  ref: c_runtime_api.h:162-172, gpu_op.cu:221-235, 1201-1233 */
 int DLGpuRelu(const DLArrayHandle input, DLArrayHandle output);
 int DLGpuReluGradient(const DLArrayHandle input, const DLArrayHandle in_grad,
                       DLArrayHandle output);
@@ -194,6 +194,13 @@ int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLArrayHandle 
                                  const DLArrayHandle filter, DLArrayHandle dinput,
                                  void ***list, void **handle, int *memorytoSaving,
                                  void **stream);
+
+/* No counterpart in the reference: introspection for benchmarks.  Writes the name
+ * of the kernel variant, tile and k-split count that conv `which` (0 forward,
+ * 1 grad-data, 2 grad-filter) launches for this descriptor, and its algorithmic
+ * flop count 2*N*K*C*R*S*P*Q. */
+int DLGpuConvolutionDescribeKernel(void ***list, int which, char *name, int name_len,
+                                   double *flops);
 
 /* ----------------------------------------------------------------- pooling */
 

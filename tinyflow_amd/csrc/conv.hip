@@ -347,7 +347,79 @@ bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
 
 constexpr int64_t kMaxBytes = (int64_t)1 << 31;  // buffer offsets are 31-bit
 
+// Launch plan of each of the three convolutions of a descriptor: which loader
+// mode / epilogue, which tile and how many k-splits.  The entry points and the
+// introspection call below both use it, so they cannot disagree.
+struct ConvPlan {
+  const char *variant;
+  int bm, bn, splits;
+  int M, N, K;
+};
+
+ConvPlan plan_forward(const ConvDesc *d) {
+  ConvPlan p;
+  p.M = d->K;
+  p.N = d->N * d->P * d->Q;
+  p.K = d->C * d->R * d->S;
+  pick_tile(p.M, p.N, p.bm, p.bn);
+  p.splits = 1;
+  p.variant = (d->pad_h || d->pad_w) ? "fwd_pad" : "fwd_nopad";
+  return p;
+}
+
+ConvPlan plan_dgrad(const ConvDesc *d) {
+  ConvPlan p;
+  const int RS = d->R * d->S;
+  p.M = d->C;
+  p.K = d->K * RS;
+  p.splits = 1;
+  if (RS == 1) {
+    p.N = d->N * d->P * d->Q;
+    pick_tile(p.M, p.N, p.bm, p.bn);
+    p.variant = (d->u == 1 && d->v == 1) ? "dgrad_1x1" : "dgrad_1x1_scatter";
+  } else {
+    p.N = d->N * d->H * d->W;
+    if (d->u == 1 && d->v == 1) {
+      pick_tile(p.M, p.N, p.bm, p.bn);
+      p.variant = "dgrad_pad";
+    } else {
+      p.bm = p.bn = 64;
+      p.variant = "dgrad_strided";
+    }
+  }
+  return p;
+}
+
+ConvPlan plan_wgrad(const ConvDesc *d) {
+  ConvPlan p;
+  p.M = d->K;
+  p.N = d->C * d->R * d->S;
+  p.K = d->N * d->P * d->Q;
+  const bool big = p.M > 64 && p.N > 64;
+  p.bm = p.bn = big ? 128 : 64;
+  const int tiles = cdiv(p.M, p.bm) * cdiv(p.N, p.bn);
+  p.splits = make_geometry(p.M, p.N, p.K, p.bm, p.bn, choose_splits(tiles, p.K, 8 * BK)).splits;
+  p.variant = (d->pad_h || d->pad_w) ? "wgrad_pad" : "wgrad_nopad";
+  return p;
+}
+
 }  // namespace
+
+// Introspection for benchmarks (no counterpart in the reference): writes a short
+// name of the kernel variant that `which` (0 forward, 1 grad-data, 2 grad-filter)
+// launches for this descriptor, e.g. "wgrad_pad_128x128_s37", and returns the
+// algorithmic flop count 2*N*K*C*R*S*P*Q through *flops.
+extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *name, int name_len,
+                                              double *flops) {
+  ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
+  TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
+  TF_REQUIRE(which >= 0 && which <= 2 && name && name_len > 0, "bad arguments");
+  const ConvPlan p = which == 0 ? plan_forward(d) : which == 1 ? plan_dgrad(d) : plan_wgrad(d);
+  snprintf(name, (size_t)name_len, "%s_%dx%d_s%d", p.variant, p.bm, p.bn, p.splits);
+  if (flops)
+    *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
+  return 0;
+}
 
 extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, const int *filter_shapes,
                                                     int *output_shapes, int dataformat, int padding,
@@ -406,10 +478,10 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
   if (check_conv_arrays(d, input, filter, output) != 0) return -1;
   if (ensure_tables(d) != 0) return -1;
   hipStream_t s = stream_of(stream);
-  const int M = d->K, N = d->N * d->P * d->Q, K = d->C * d->R * d->S;
+  const ConvPlan plan = plan_forward(d);
+  const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
-  int bm, bn;
-  pick_tile(M, N, bm, bn);
+  const int bm = plan.bm, bn = plan.bn;
   const Geometry g = make_geometry(M, N, K, bm, bn, 1);
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
   with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
@@ -441,8 +513,8 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   if (ensure_tables(d) != 0) return -1;
   hipStream_t s = stream_of(stream);
   const int RS = d->R * d->S;
-  const int M = d->C;
-  const int K = d->K * RS;
+  const ConvPlan plan = plan_dgrad(d);
+  const int M = plan.M, K = plan.K;
   if (numel(dinput) == 0) return 0;
   if (numel(doutput) == 0) return DLGpuArraySet(dinput, 0.f, stream);
 
@@ -466,9 +538,8 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
 
   if (RS == 1) {
     // 1x1 filter (pad 0): compact GEMM over the output pixels + scatter
-    const int N = d->N * PQ;
-    int bm, bn;
-    pick_tile(M, N, bm, bn);
+    const int N = plan.N;
+    const int bm = plan.bm, bn = plan.bn;
     const Geometry g = make_geometry(M, N, K, bm, bn, 1);
     with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
       constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value;
@@ -486,10 +557,9 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
       }
     });
   } else {
-    const int N = d->N * d->H * d->W;
+    const int N = plan.N;
     const int HW = d->H * d->W;
-    int bm, bn;
-    pick_tile(M, N, bm, bn);
+    const int bm = plan.bm, bn = plan.bn;
     StoreNCHW ep{(float *)dinput->data, M, N, FastDiv((uint32_t)HW), HW};
     if (d->u == 1 && d->v == 1) {
       const Geometry g = make_geometry(M, N, K, bm, bn, 1);
@@ -525,14 +595,13 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
   TF_REQUIRE(on_gpu(dfilter) && same_shape(dfilter, filter), "dfilter must have the filter's shape");
   hipStream_t s = stream_of(stream);
   const int PQ = d->P * d->Q, RS = d->R * d->S;
-  const int M = d->K, N = d->C * RS, K = d->N * PQ;
+  const ConvPlan plan = plan_wgrad(d);
+  const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
   if (K == 0) return DLGpuArraySet(dfilter, 0.f, stream);
 
-  const bool big = M > 64 && N > 64;
-  const int bm = big ? 128 : 64, bn = big ? 128 : 64;
-  const int tiles = cdiv(M, bm) * cdiv(N, bn);
-  Geometry g = make_geometry(M, N, K, bm, bn, choose_splits(tiles, K, 8 * BK));
+  const int bm = plan.bm, bn = plan.bn;
+  Geometry g = make_geometry(M, N, K, bm, bn, plan.splits);
   float *dst = (float *)dfilter->data;
   float *partial = nullptr;
   if (g.splits > 1) {
