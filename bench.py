@@ -86,12 +86,17 @@ class ConvTimer(object):
         key = (ctypes.addressof(cudnnlist.contents), which)
         hit = self._describe_cache.get(key)
         if hit is None:
-            buf = ctypes.create_string_buffer(96)
+            buf = ctypes.create_string_buffer(256)
             flops = ctypes.c_double()
-            rc = self.lib.DLGpuConvolutionDescribeKernel(cudnnlist, which, buf, 96, ctypes.byref(flops))
+            rc = self.lib.DLGpuConvolutionDescribeKernel(cudnnlist, which, buf, 256, ctypes.byref(flops))
             if rc != 0:
                 raise RuntimeError("DLGpuConvolutionDescribeKernel failed")
-            hit = (buf.value.decode(), flops.value)
+            # group by kernel symbol; calls whose reduction is split also run the
+            # small partial-sum kernel inside the bracketed region, so they are
+            # kept apart from the single-kernel calls
+            variant, symbol = buf.value.decode().split(" | ")
+            split = not variant.endswith(" s1")
+            hit = ((symbol + " + split_sum_kernel") if split else symbol, flops.value)
             self._describe_cache[key] = hit
         return hit
 

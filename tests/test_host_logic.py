@@ -62,11 +62,11 @@ def test_conv_out_shape_descriptor(case):
     ph, pw = O.conv_pad(w_shape[2], padding), O.conv_pad(w_shape[3], padding)
     assert out == (x_shape[0], w_shape[0], O.conv_out_extent(x_shape[2], w_shape[2], ph, u),
                    O.conv_out_extent(x_shape[3], w_shape[3], pw, v))
-    name = ctypes.create_string_buffer(96)
+    name = ctypes.create_string_buffer(256)
     flops = ctypes.c_double()
     for which in range(3):
-        assert _LIB.DLGpuConvolutionDescribeKernel(lst, which, name, 96, ctypes.byref(flops)) == 0
-        assert name.value
+        assert _LIB.DLGpuConvolutionDescribeKernel(lst, which, name, 256, ctypes.byref(flops)) == 0
+        assert b" | gemm_kernel<" in name.value
         expect = 2.0 * np.prod(out, dtype=np.float64) * w_shape[1] * w_shape[2] * w_shape[3]
         assert flops.value == expect
 

@@ -21,44 +21,46 @@
 #include "gemm_core.h"
 #include "internal.h"
 
-#include <mutex>
 #include <type_traits>
-#include <vector>
 
 using namespace tf;
 using namespace tf::gemm;
 
 namespace {
 
-inline int pack_taps(int dy, int dx) { return (int)(((uint32_t)(dy & 0xffff) << 16) | (uint32_t)(dx & 0xffff)); }
-__device__ inline int tap_y(int packed) { return packed >> 16; }                 // sign-extending
-__device__ inline int tap_x(int packed) { return (int)(short)(packed & 0xffff); }
 
 // ---- gathered operand, lanes along the pixel index ------------------------------
 // element(pixel, k): source tensor T[img][ch][Hs][Ws], pixel -> (img, oy, ox),
-// k -> (ch, dy, dx) through a table; reads T[img][ch][oy*sy+by+dy][ox*sx+bx+dx].
+// k -> (ch, r, s) with (dy, dx) = dir * (r, s); reads T[img][ch][oy*sy+by+dy][ox*sx+bx+dx].
 // MODE 0: taps are always inside the image (no padding)      -> no range test
 // MODE 1: range test (zero padding)
 // MODE 2: additionally the tapped coordinate must be divisible by the conv
 //         stride and is divided by it (grad-data of a strided filter larger than 1x1)
-template <int D, int MODE>
+template <int D, int BK, int MODE>
 struct GatherAlong {
-  using Map = AlongMap<D>;
+  using Map = AlongMap<D, BK>;
   static constexpr int EPT = Map::EPT;
   const float *base;
   uint32_t bytes;
-  const int2 *tab;  // [k_extent]: .x = ch * Hs * Ws, .y = packed (dy, dx)
   int k_extent, n_extent;
+  FastDiv div_rs, div_s;     // k -> (ch, r, s): ch = k / (R*S), r = (k % (R*S)) / S
+  int ch_stride;             // Hs * Ws
   FastDiv div_img, div_row;  // pixels per image, pixels per row
   int img_stride;            // elements per image of T
   int Hs, Ws;
   int sy, sx, by, bx;
+  int dir;                   // +1: dy = r, dx = s (forward); -1: dy = -r, dx = -s (grad-data)
+  int R, S;
   FastDiv div_u, div_v;      // MODE 2 only
 
   struct State {
     Map map;
     __amdgpu_buffer_rsrc_t rsrc;
-    int img_off, y0, x0;
+    // MODE 0/1: byte offset of (img, y0, x0), OOB for a lane past the last pixel;
+    // bit r of row_ok / bit s of col_ok says whether tap row r / column s lands
+    // inside the image for this lane's pixel (the pixel is fixed for the whole kernel)
+    uint32_t lane_off, row_ok, col_ok;
+    int img_off, y0, x0;  // MODE 2
     bool ok;
   };
   __device__ inline void init(State &st, int origin, int tid) const {
@@ -72,27 +74,57 @@ struct GatherAlong {
     st.img_off = (int)img * img_stride;
     st.y0 = (int)oy * sy + by;
     st.x0 = (int)ox * sx + bx;
+    st.lane_off = st.ok ? (uint32_t)(st.img_off + st.y0 * Ws + st.x0) * 4u : OOB;
+    st.row_ok = st.col_ok = 0;
+    if (MODE == 1 && st.ok) {
+      for (int r = 0; r < R; ++r)
+        if ((uint32_t)(st.y0 + dir * r) < (uint32_t)Hs) st.row_ok |= 1u << r;
+      for (int s = 0; s < S; ++s)
+        if ((uint32_t)(st.x0 + dir * s) < (uint32_t)Ws) st.col_ok |= 1u << s;
+    }
   }
-  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
+    // k is wave-uniform, so its decomposition into (channel, tap row, tap column)
+    // is scalar arithmetic: no memory access stands between one stage and the
+    // next, and validity is folded into the offset's top bit instead of being
+    // branched on -- the stage is straight-line code.
+    struct Tap { int x, r, s; } t[EPT];
+    uint32_t k_bad[EPT];
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
-      const int k = k0 + st.map.k_of(e);       // wave-uniform
-      const bool k_ok = k < k_extent;
-      const int2 t = tab[k_ok ? k : 0];
-      int yy = st.y0 + tap_y(t.y), xx = st.x0 + tap_x(t.y);
-      bool ok = st.ok && k_ok;
-      if (MODE == 2) {
-        ok = ok && yy >= 0 && xx >= 0;
+      const int k = k0 + st.map.k_of(e);
+      const uint32_t kc = (uint32_t)min(k, k_extent - 1);
+      uint32_t ch, rs, r, s;
+      div_rs.divmod(kc, ch, rs);
+      div_s.divmod(rs, r, s);
+      t[e].r = (int)r;
+      t[e].s = (int)s;
+      t[e].x = (int)ch * ch_stride + dir * ((int)r * Ws + (int)s);
+      k_bad[e] = k < k_limit ? 0u : OOB;
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      if (MODE == 0) {
+        // no padding: every tap of a valid pixel is inside the image
+        reg[e] = buf_load(st.rsrc, (st.lane_off + (uint32_t)t[e].x * 4u) | k_bad[e]);
+      } else if (MODE == 1) {
+        const uint32_t tap_bad = ~((st.row_ok >> t[e].r) & (st.col_ok >> t[e].s)) << 31;
+        reg[e] = buf_load(st.rsrc, (st.lane_off + (uint32_t)t[e].x * 4u) | tap_bad | k_bad[e]);
+      } else {
+        // strided filter larger than 1x1 (grad-data only): the tapped coordinate
+        // must be divisible by the stride and is divided by it
+        const int r = t[e].r, s = t[e].s;
+        const int yy = st.y0 - r, xx = st.x0 - s;
+        bool ok = st.ok && yy >= 0 && xx >= 0;
         uint32_t qy, ry, qx, rx;
         div_u.divmod((uint32_t)(yy < 0 ? 0 : yy), qy, ry);
         div_v.divmod((uint32_t)(xx < 0 ? 0 : xx), qx, rx);
-        ok = ok && ry == 0 && rx == 0;
-        yy = (int)qy;
-        xx = (int)qx;
+        ok = ok && ry == 0 && rx == 0 && qy < (uint32_t)Hs && qx < (uint32_t)Ws;
+        // t.x = ch*Hs*Ws - r*Ws - s: add the taps back to get the channel offset
+        const int ch_off = t[e].x + r * Ws + s;
+        const uint32_t off = (uint32_t)(st.img_off + ch_off + (int)qy * Ws + (int)qx) * 4u;
+        reg[e] = buf_load(st.rsrc, (ok ? off : OOB) | k_bad[e]);
       }
-      if (MODE != 0) ok = ok && (uint32_t)yy < (uint32_t)Hs && (uint32_t)xx < (uint32_t)Ws;
-      const uint32_t off = (uint32_t)(st.img_off + t.x + yy * Ws + xx) * 4u;
-      reg[e] = buf_load(st.rsrc, ok ? off : OOB);
     }
   }
   template <int LD>
@@ -105,9 +137,9 @@ struct GatherAlong {
 // ---- gathered operand, lanes along the reduction (grad-filter's x) --------------
 // element(col, k): col -> (c, r, s) fixed per lane for the whole kernel,
 // k -> (img, p, q) recomputed per stage; reads x[img][c][p*u+r-pad_h][q*v+s-pad_w].
-template <int D, int MODE>
+template <int D, int BK, int MODE>
 struct GatherAcross {
-  using Map = AcrossMap<D>;
+  using Map = AcrossMap<D, BK>;
   static constexpr int EPT = Map::EPT;
   const float *base;
   uint32_t bytes;
@@ -136,9 +168,9 @@ struct GatherAcross {
       st.taps[e] = (int)((r << 16) | s);
     }
   }
-  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
     const int kidx = k0 + st.map.k_local;
-    const bool k_ok = kidx < k_extent;
+    const bool k_ok = kidx < k_limit;
     uint32_t img, rem, p, q;
     div_pq.divmod((uint32_t)(k_ok ? kidx : 0), img, rem);
     div_q.divmod(rem, p, q);
@@ -161,9 +193,9 @@ struct GatherAcross {
 };
 
 // ---- grad-filter's dy operand: element(m = out channel, k = (img, pq)) -----------
-template <int D>
+template <int D, int BK>
 struct DyAcross {
-  using Map = AcrossMap<D>;
+  using Map = AcrossMap<D, BK>;
   static constexpr int EPT = Map::EPT;
   const float *base;
   uint32_t bytes;
@@ -185,9 +217,9 @@ struct DyAcross {
       st.row_off[e] = m < m_extent ? (uint32_t)m * (uint32_t)PQ * 4u : OOB;
     }
   }
-  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
     const int kidx = k0 + st.map.k_local;
-    const bool k_ok = kidx < k_extent;
+    const bool k_ok = kidx < k_limit;
     uint32_t img, pq;
     div_pq.divmod((uint32_t)(k_ok ? kidx : 0), img, pq);
     const uint32_t k_off = k_ok ? (uint32_t)((int)img * img_stride + (int)pq) * 4u : OOB;
@@ -209,11 +241,14 @@ struct StoreNCHW {
   int m_extent, n_extent;
   FastDiv div_hw;
   int HW;
+  int64_t split_stride;  // elements between the partial outputs of consecutive k-splits
   struct State {
+    float *base;
     int col_base[4];  // img * CH * HW + pixel, or -1
   };
   template <int TN>
-  __device__ inline void init(State &st, int n_wave, int lane, int /*split*/) const {
+  __device__ inline void init(State &st, int n_wave, int lane, int split) const {
+    st.base = out + (int64_t)split * split_stride;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n_wave + 32 * j + (lane & 31);
@@ -223,7 +258,7 @@ struct StoreNCHW {
     }
   }
   __device__ inline void store(const State &st, int m, int /*n*/, int j, float v) const {
-    if (m < m_extent && st.col_base[j] >= 0) out[st.col_base[j] + m * HW] = v;
+    if (m < m_extent && st.col_base[j] >= 0) st.base[st.col_base[j] + m * HW] = v;
   }
 };
 
@@ -280,11 +315,16 @@ __global__ __launch_bounds__(256) void filter_to_krsc_kernel(const float *__rest
 template <int V>
 using IC = std::integral_constant<int, V>;
 
+// Tile shapes and the stage depth that goes with each (measured): 16-deep stages
+// for the wide tiles, 32-deep for the 64 x 64 tile, whose per-stage overhead is
+// otherwise as large as its eight MFMAs per wave.
+inline int stage_depth(int bm, int bn) { return (bm == 64 && bn == 64) ? 32 : 16; }
+
 template <class F>
 void with_tile(int bm, int bn, F &&f) {
-  if (bm == 128 && bn == 128) f(IC<128>{}, IC<128>{});
-  else if (bm == 64 && bn == 128) f(IC<64>{}, IC<128>{});
-  else f(IC<64>{}, IC<64>{});
+  if (bm == 128 && bn == 128) f(IC<128>{}, IC<128>{}, IC<16>{});
+  else if (bm == 64 && bn == 128) f(IC<64>{}, IC<128>{}, IC<16>{});
+  else f(IC<64>{}, IC<64>{}, IC<32>{});
 }
 
 // Largest tile that still yields about 1.5 workgroups per CU; the smallest otherwise.
@@ -299,46 +339,10 @@ void pick_tile(int M, int N, int &bm, int &bn) {
   }
 }
 
-template <int BM, int BN, class AL, class BL, class EP>
+template <int BM, int BN, int BK, class AL, class BL, class EP>
 void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s) {
-  hipLaunchKernelGGL((gemm_kernel<BM, BN, AL, BL, EP>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl, ep, K,
-                     g.k_per_split, g.tiles_m, g.tiles_n);
-}
-
-std::mutex g_tab_mu;
-
-int upload_table(const std::vector<int> &host, int **dev) {
-  TF_HIP(hipMalloc((void **)dev, host.size() * sizeof(int)));
-  TF_HIP(hipMemcpy(*dev, host.data(), host.size() * sizeof(int), hipMemcpyHostToDevice));
-  return 0;
-}
-
-// Reduction-index tables of a descriptor, built on first use and kept for its lifetime.
-int ensure_tables(ConvDesc *d) {
-  std::lock_guard<std::mutex> g(g_tab_mu);
-  if (!d->fwd_tab) {
-    std::vector<int> t((size_t)d->C * d->R * d->S * 2);
-    size_t i = 0;
-    for (int c = 0; c < d->C; ++c)
-      for (int r = 0; r < d->R; ++r)
-        for (int s = 0; s < d->S; ++s) {
-          t[i++] = c * d->H * d->W;
-          t[i++] = pack_taps(r, s);
-        }
-    if (upload_table(t, &d->fwd_tab) != 0) return -1;
-  }
-  if (!d->dgrad_tab) {
-    std::vector<int> t((size_t)d->K * d->R * d->S * 2);
-    size_t i = 0;
-    for (int k = 0; k < d->K; ++k)
-      for (int r = 0; r < d->R; ++r)
-        for (int s = 0; s < d->S; ++s) {
-          t[i++] = k * d->P * d->Q;
-          t[i++] = pack_taps(-r, -s);
-        }
-    if (upload_table(t, &d->dgrad_tab) != 0) return -1;
-  }
-  return 0;
+  hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl, ep,
+                     K, g.k_per_split, g.tiles_m, g.tiles_n);
 }
 
 bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
@@ -351,10 +355,21 @@ constexpr int64_t kMaxBytes = (int64_t)1 << 31;  // buffer offsets are 31-bit
 // mode / epilogue, which tile and how many k-splits.  The entry points and the
 // introspection call below both use it, so they cannot disagree.
 struct ConvPlan {
-  const char *variant;
+  const char *variant;   // short name of the loader / epilogue combination
+  const char *a_loader, *b_loader, *epilogue;  // as they appear in the kernel symbol
+  int b_mode;            // MODE template argument of the gathered operand, -1 if none
   int bm, bn, splits;
   int M, N, K;
 };
+
+// Forward and grad-data may also split the reduction when the output has too few
+// tiles to fill the chip and the reduction is long (the 14x14 and 7x7 stages):
+// each split writes a partial output that a fixed-order pass adds up.
+int splits_for_output(const ConvPlan &p) {
+  const int tiles = cdiv(p.M, p.bm) * cdiv(p.N, p.bn);
+  int splits = choose_splits(tiles, p.K, 512);
+  return splits > 4 ? 4 : splits;
+}
 
 ConvPlan plan_forward(const ConvDesc *d) {
   ConvPlan p;
@@ -362,8 +377,12 @@ ConvPlan plan_forward(const ConvDesc *d) {
   p.N = d->N * d->P * d->Q;
   p.K = d->C * d->R * d->S;
   pick_tile(p.M, p.N, p.bm, p.bn);
-  p.splits = 1;
+  p.splits = splits_for_output(p);
   p.variant = (d->pad_h || d->pad_w) ? "fwd_pad" : "fwd_nopad";
+  p.a_loader = "PlainAcross";
+  p.b_loader = "GatherAlong";
+  p.epilogue = "StoreNCHW";
+  p.b_mode = (d->pad_h || d->pad_w) ? 1 : 0;
   return p;
 }
 
@@ -373,18 +392,27 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   p.M = d->C;
   p.K = d->K * RS;
   p.splits = 1;
+  p.a_loader = "PlainAlong";
+  p.b_loader = "GatherAlong";
+  p.epilogue = "StoreNCHW";
+  p.b_mode = 0;
   if (RS == 1) {
     p.N = d->N * d->P * d->Q;
     pick_tile(p.M, p.N, p.bm, p.bn);
     p.variant = (d->u == 1 && d->v == 1) ? "dgrad_1x1" : "dgrad_1x1_scatter";
+    if (d->u == 1 && d->v == 1) p.splits = splits_for_output(p);
+    else p.epilogue = "StoreScatter";
   } else {
     p.N = d->N * d->H * d->W;
     if (d->u == 1 && d->v == 1) {
       pick_tile(p.M, p.N, p.bm, p.bn);
+      p.splits = splits_for_output(p);
       p.variant = "dgrad_pad";
+      p.b_mode = 1;
     } else {
       p.bm = p.bn = 64;
       p.variant = "dgrad_strided";
+      p.b_mode = 2;
     }
   }
   return p;
@@ -398,73 +426,34 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   const bool big = p.M > 64 && p.N > 64;
   p.bm = p.bn = big ? 128 : 64;
   const int tiles = cdiv(p.M, p.bm) * cdiv(p.N, p.bn);
-  p.splits = make_geometry(p.M, p.N, p.K, p.bm, p.bn, choose_splits(tiles, p.K, 8 * BK)).splits;
+  p.splits = make_geometry(p.M, p.N, p.K, p.bm, p.bn, choose_splits(tiles, p.K, 256), stage_depth(p.bm, p.bn)).splits;
   p.variant = (d->pad_h || d->pad_w) ? "wgrad_pad" : "wgrad_nopad";
+  p.a_loader = "DyAcross";
+  p.b_loader = "GatherAcross";
+  p.epilogue = "StoreRowMajor";
+  p.b_mode = (d->pad_h || d->pad_w) ? 1 : 0;
   return p;
 }
 
 }  // namespace
 
-// Introspection for benchmarks (no counterpart in the reference): writes a short
-// name of the kernel variant that `which` (0 forward, 1 grad-data, 2 grad-filter)
-// launches for this descriptor, e.g. "wgrad_pad_128x128_s37", and returns the
-// algorithmic flop count 2*N*K*C*R*S*P*Q through *flops.
+// Introspection for benchmarks (no counterpart in the reference): describes the
+// kernel that `which` (0 forward, 1 grad-data, 2 grad-filter) launches for this
+// descriptor as "<variant> <bm>x<bn> s<splits> | <kernel symbol>", where the symbol
+// is spelled the way a profiler prints it (anonymous-namespace qualifiers
+// dropped), and returns the algorithmic flop count 2*N*K*C*R*S*P*Q through *flops.
 extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *name, int name_len,
                                               double *flops) {
   ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
   TF_REQUIRE(which >= 0 && which <= 2 && name && name_len > 0, "bad arguments");
   const ConvPlan p = which == 0 ? plan_forward(d) : which == 1 ? plan_dgrad(d) : plan_wgrad(d);
-  snprintf(name, (size_t)name_len, "%s_%dx%d_s%d", p.variant, p.bm, p.bn, p.splits);
+  const int bk = stage_depth(p.bm, p.bn);
+  snprintf(name, (size_t)name_len,
+           "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d>, %s<%d, %d, %d>, %s>", p.variant, p.bm, p.bn,
+           p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, p.b_loader, p.bn, bk, p.b_mode, p.epilogue);
   if (flops)
     *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
-  return 0;
-}
-
-extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, const int *filter_shapes,
-                                                    int *output_shapes, int dataformat, int padding,
-                                                    const int u, const int v, void ***list) {
-  TF_REQUIRE(input_shapes && filter_shapes && output_shapes && list, "null argument");
-  TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
-  TF_REQUIRE(u >= 1 && v >= 1, "strides must be positive");
-  ConvDesc *d = new ConvDesc();
-  d->magic = kMagicConv;
-  d->N = input_shapes[0];
-  d->C = input_shapes[1];
-  d->H = input_shapes[2];
-  d->W = input_shapes[3];
-  d->K = filter_shapes[0];
-  d->R = filter_shapes[2];
-  d->S = filter_shapes[3];
-  TF_REQUIRE(filter_shapes[1] == d->C, "filter expects %d input channels, input has %d", filter_shapes[1], d->C);
-  d->pad_h = padding == 1 ? d->R / 2 : 0;  // "SAME" is a symmetric k/2, "VALID" is 0
-  d->pad_w = padding == 1 ? d->S / 2 : 0;
-  d->u = u;
-  d->v = v;
-  TF_REQUIRE(d->H + 2 * d->pad_h >= d->R && d->W + 2 * d->pad_w >= d->S, "filter larger than padded input");
-  d->P = 1 + (d->H + 2 * d->pad_h - d->R) / u;
-  d->Q = 1 + (d->W + 2 * d->pad_w - d->S) / v;
-  TF_REQUIRE(d->R < 32768 && d->S < 32768, "filter extent too large");
-  d->fwd_tab = nullptr;
-  d->dgrad_tab = nullptr;
-  output_shapes[0] = d->N;
-  output_shapes[1] = d->K;
-  output_shapes[2] = d->P;
-  output_shapes[3] = d->Q;
-  // four slots like the reference's {x, w, conv, y} descriptor list
-  void **slots = (void **)malloc(sizeof(void *) * 4);
-  for (int i = 0; i < 4; ++i) slots[i] = d;
-  *list = slots;
-  return 0;
-}
-
-static int check_conv_arrays(const ConvDesc *d, const DLArray *x, const DLArray *w, const DLArray *y) {
-  TF_REQUIRE(on_gpu(x) && on_gpu(w) && on_gpu(y), "arrays must live on the GPU");
-  TF_REQUIRE(shape_is(x, d->N, d->C, d->H, d->W), "input does not match the descriptor (N,C,H,W)");
-  TF_REQUIRE(shape_is(w, d->K, d->C, d->R, d->S), "filter does not match the descriptor (K,C,R,S)");
-  TF_REQUIRE(shape_is(y, d->N, d->K, d->P, d->Q), "output does not match the descriptor (N,K,P,Q)");
-  TF_REQUIRE(numel(x) * 4 < kMaxBytes && numel(y) * 4 < kMaxBytes && numel(w) * 4 < kMaxBytes,
-             "tensors of 2 GiB or more are not supported");
   return 0;
 }
 
@@ -472,33 +461,45 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
                                          DLArrayHandle output, void ***list, void **handle,
                                          int *memorytoSaving, void **stream) {
   (void)handle;
-  (void)memorytoSaving;
   ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
   if (check_conv_arrays(d, input, filter, output) != 0) return -1;
-  if (ensure_tables(d) != 0) return -1;
   hipStream_t s = stream_of(stream);
   const ConvPlan plan = plan_forward(d);
   const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
   const int bm = plan.bm, bn = plan.bn;
-  const Geometry g = make_geometry(M, N, K, bm, bn, 1);
+  const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+  float *partial = nullptr;
+  if (g.splits > 1) {
+    const size_t bytes = (size_t)g.splits * numel(output) * sizeof(float);
+    partial = (float *)device_alloc(bytes);
+    if (!partial) {
+      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      return 0;
+    }
+  }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
-  with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
-    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value;
-    PlainAcross<BM> al{(const float *)filter->data, (uint32_t)(numel(filter) * 4), K, M, K};
-    StoreNCHW ep{(float *)output->data, M, N, FastDiv((uint32_t)(d->P * d->Q)), d->P * d->Q};
+  with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
+    PlainAcross<BM, BK> al{(const float *)filter->data, (uint32_t)(numel(filter) * 4), K, M, K};
+    StoreNCHW ep{partial ? partial : (float *)output->data, M, N, FastDiv((uint32_t)(d->P * d->Q)),
+                 d->P * d->Q, numel(output)};
     auto run = [&](auto mode_c) {
       constexpr int MODE = decltype(mode_c)::value;
-      GatherAlong<BN, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4),
-                               (const int2 *)d->fwd_tab, K, N,
+      GatherAlong<BN, BK, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4), K, N,
+                               FastDiv((uint32_t)(d->R * d->S)), FastDiv((uint32_t)d->S), d->H * d->W,
                                FastDiv((uint32_t)(d->P * d->Q)), FastDiv((uint32_t)d->Q),
                                d->C * d->H * d->W, d->H, d->W, d->u, d->v, -d->pad_h, -d->pad_w,
-                               FastDiv(1), FastDiv(1)};
-      launch<BM, BN>(al, bl, ep, K, g, s);
+                               1, d->R, d->S, FastDiv(1), FastDiv(1)};
+      launch<BM, BN, BK>(al, bl, ep, K, g, s);
     };
     if (padded) run(IC<1>{}); else run(IC<0>{});
   });
+  if (partial) {
+    launch_split_sum(partial, (float *)output->data, numel(output), g.splits, s);
+    device_free(partial);
+  }
   return finish(s, "DLGpuConvolution2DForward");
 }
 
@@ -510,7 +511,6 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
   if (check_conv_arrays(d, input, filter, doutput) != 0) return -1;
   TF_REQUIRE(on_gpu(dinput) && same_shape(dinput, input), "dinput must have the input's shape");
-  if (ensure_tables(d) != 0) return -1;
   hipStream_t s = stream_of(stream);
   const int RS = d->R * d->S;
   const ConvPlan plan = plan_dgrad(d);
@@ -535,51 +535,70 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   }
   const uint32_t w_bytes = (uint32_t)(numel(filter) * 4), dy_bytes = (uint32_t)(numel(doutput) * 4);
   const int PQ = d->P * d->Q;
+  float *partial = nullptr;
+  if (plan.splits > 1) {
+    const size_t bytes = (size_t)plan.splits * numel(dinput) * sizeof(float);
+    partial = (float *)device_alloc(bytes);
+    if (!partial) {
+      if (wt_scratch) device_free(wt_scratch);
+      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      return 0;
+    }
+  }
+  float *dst = partial ? partial : (float *)dinput->data;
+  const int64_t dx_count = numel(dinput);
 
   if (RS == 1) {
     // 1x1 filter (pad 0): compact GEMM over the output pixels + scatter
     const int N = plan.N;
     const int bm = plan.bm, bn = plan.bn;
-    const Geometry g = make_geometry(M, N, K, bm, bn, 1);
-    with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
-      constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value;
-      PlainAlong<BM> al{wt, w_bytes, d->C, M, K};
-      GatherAlong<BN, 0> bl{(const float *)doutput->data, dy_bytes, (const int2 *)d->dgrad_tab, K, N,
+    const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+    with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+      constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
+      PlainAlong<BM, BK> al{wt, w_bytes, d->C, M, K};
+      GatherAlong<BN, BK, 0> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv(1), FastDiv(1), PQ,
                             FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), d->K * PQ, d->P, d->Q,
-                            1, 1, 0, 0, FastDiv(1), FastDiv(1)};
+                            1, 1, 0, 0, -1, 1, 1, FastDiv(1), FastDiv(1)};
       if (d->u == 1 && d->v == 1) {
-        StoreNCHW ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), PQ};
-        launch<BM, BN>(al, bl, ep, K, g, s);
+        StoreNCHW ep{dst, M, N, FastDiv((uint32_t)PQ), PQ, dx_count};
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
       } else {
         StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
                         d->H, d->W, d->u, d->v};
-        launch<BM, BN>(al, bl, ep, K, g, s);
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
       }
     });
   } else {
     const int N = plan.N;
     const int HW = d->H * d->W;
     const int bm = plan.bm, bn = plan.bn;
-    StoreNCHW ep{(float *)dinput->data, M, N, FastDiv((uint32_t)HW), HW};
+    StoreNCHW ep{dst, M, N, FastDiv((uint32_t)HW), HW, dx_count};
     if (d->u == 1 && d->v == 1) {
-      const Geometry g = make_geometry(M, N, K, bm, bn, 1);
-      with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
-        constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value;
-        PlainAlong<BM> al{wt, w_bytes, d->C, M, K};
-        GatherAlong<BN, 1> bl{(const float *)doutput->data, dy_bytes, (const int2 *)d->dgrad_tab, K, N,
+      const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+      with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+        constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
+        PlainAlong<BM, BK> al{wt, w_bytes, d->C, M, K};
+        GatherAlong<BN, BK, 1> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv((uint32_t)RS),
+                              FastDiv((uint32_t)d->S), PQ,
                               FastDiv((uint32_t)HW), FastDiv((uint32_t)d->W), d->K * PQ, d->P, d->Q,
-                              1, 1, d->pad_h, d->pad_w, FastDiv(1), FastDiv(1)};
-        launch<BM, BN>(al, bl, ep, K, g, s);
+                              1, 1, d->pad_h, d->pad_w, -1, d->R, d->S, FastDiv(1), FastDiv(1)};
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
       });
     } else {
       // strided filter larger than 1x1: every input pixel, taps filtered by divisibility
-      const Geometry g = make_geometry(M, N, K, 64, 64, 1);
-      PlainAlong<64> al{wt, w_bytes, d->C, M, K};
-      GatherAlong<64, 2> bl{(const float *)doutput->data, dy_bytes, (const int2 *)d->dgrad_tab, K, N,
+      const Geometry g = make_geometry(M, N, K, 64, 64, 1, 32);
+      PlainAlong<64, 32> al{wt, w_bytes, d->C, M, K};
+      GatherAlong<64, 32, 2> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv((uint32_t)RS),
+                            FastDiv((uint32_t)d->S), PQ,
                             FastDiv((uint32_t)HW), FastDiv((uint32_t)d->W), d->K * PQ, d->P, d->Q,
-                            1, 1, d->pad_h, d->pad_w, FastDiv((uint32_t)d->u), FastDiv((uint32_t)d->v)};
-      launch<64, 64>(al, bl, ep, K, g, s);
+                            1, 1, d->pad_h, d->pad_w, -1, d->R, d->S,
+                            FastDiv((uint32_t)d->u), FastDiv((uint32_t)d->v)};
+      launch<64, 64, 32>(al, bl, ep, K, g, s);
     }
+  }
+  if (partial) {
+    launch_split_sum(partial, (float *)dinput->data, dx_count, plan.splits, s);
+    device_free(partial);
   }
   if (wt_scratch) device_free(wt_scratch);
   return finish(s, "DLGpuConvolutionBackwardData");
@@ -601,7 +620,7 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
   if (K == 0) return DLGpuArraySet(dfilter, 0.f, stream);
 
   const int bm = plan.bm, bn = plan.bn;
-  Geometry g = make_geometry(M, N, K, bm, bn, plan.splits);
+  Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
   float *dst = (float *)dfilter->data;
   float *partial = nullptr;
   if (g.splits > 1) {
@@ -614,19 +633,19 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
     dst = partial;
   }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
-  with_tile(bm, bn, [&](auto bm_c, auto bn_c) {
-    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value;
+  with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     if constexpr (BM == BN) {  // only the square tiles are used for grad-filter
-      DyAcross<BM> al{(const float *)doutput->data, (uint32_t)(numel(doutput) * 4), K, M,
+      DyAcross<BM, BK> al{(const float *)doutput->data, (uint32_t)(numel(doutput) * 4), K, M,
                       FastDiv((uint32_t)PQ), d->K * PQ, PQ};
       StoreRowMajor ep{dst, N, M, N, (int64_t)M * N};
       auto run = [&](auto mode_c) {
         constexpr int MODE = decltype(mode_c)::value;
-        GatherAcross<BN, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4), K, N,
+        GatherAcross<BN, BK, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4), K, N,
                                   FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), FastDiv((uint32_t)RS),
                                   FastDiv((uint32_t)d->S), d->C * d->H * d->W, d->H * d->W,
                                   d->H, d->W, d->u, d->v, d->pad_h, d->pad_w};
-        launch<BM, BN>(al, bl, ep, K, g, s);
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
       };
       if (padded) run(IC<1>{}); else run(IC<0>{});
     }

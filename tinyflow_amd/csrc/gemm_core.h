@@ -4,7 +4,8 @@
 //   D[m, n] = sum_k A(m, k) * B(k, n)
 //
 // One 256-lane workgroup (four wave64 waves in a 2 x 2 arrangement) owns a
-// BM x BN tile of D and walks the reduction in steps of BK = 16.  Operand tiles
+// BM x BN tile of D and walks the reduction in steps of BK (16 or 32, a template
+// parameter chosen with the tile shape).  Operand tiles
 // are fetched with bounds-checked buffer loads (an out-of-range or padded
 // element is given an offset beyond the buffer and reads as zero, so tails and
 // convolution padding need no branches), staged through double-buffered LDS as
@@ -25,7 +26,6 @@ namespace gemm {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 16;          // reduction depth of one LDS stage
 constexpr int THREADS = 256;    // four waves
 constexpr int LDS_PAD = 4;      // row padding of the LDS planes (floats)
 constexpr uint32_t OOB = 0x80000000u;  // byte offset that every buffer bound check rejects
@@ -60,7 +60,7 @@ struct FastDiv {
 // ---- thread -> tile-element maps ---------------------------------------------
 // "Along" map: the 256 lanes run along the tile's m (or n) extent D, so that one
 // load instruction of a wave reads 64 consecutive m for a single, wave-uniform k.
-template <int D>
+template <int D, int BK>
 struct AlongMap {
   static_assert(D == 64 || D == 128 || D == 256, "tile extent");
   static constexpr int KSTEP = THREADS / D;  // k rows covered per pass
@@ -74,12 +74,12 @@ struct AlongMap {
   __device__ inline int k_of(int e) const { return k_first + e * KSTEP; }
 };
 
-// "Across" map: 16 consecutive lanes run along k (the contiguous direction of
-// the operand in memory), the remaining 16 lane groups along the tile extent.
-template <int D>
+// "Across" map: BK consecutive lanes run along k (the contiguous direction of
+// the operand in memory), the remaining lane groups along the tile extent.
+template <int D, int BK>
 struct AcrossMap {
-  static_assert(D % 16 == 0, "tile extent");
-  static constexpr int DSTEP = THREADS / BK;  // 16
+  static_assert(D % (THREADS / BK) == 0, "tile extent");
+  static constexpr int DSTEP = THREADS / BK;
   static constexpr int EPT = D / DSTEP;
   int k_local;
   int d_first;
@@ -92,9 +92,9 @@ struct AcrossMap {
 
 // ---- plain row-major matrix operands -------------------------------------------
 // element(d, k) = base[k * ld + d]        (tile extent contiguous in memory)
-template <int D>
+template <int D, int BK>
 struct PlainAlong {
-  using Map = AlongMap<D>;
+  using Map = AlongMap<D, BK>;
   static constexpr int EPT = Map::EPT;
   const float *base;
   uint32_t bytes;
@@ -111,11 +111,12 @@ struct PlainAlong {
     const int d = origin + st.map.d_local;
     st.d_off = d < d_extent ? (uint32_t)d * 4u : OOB;
   }
-  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+  // k_limit: first reduction index this workgroup must not read (<= k_extent)
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
       const int k = k0 + st.map.k_of(e);
-      const uint32_t off = k < k_extent ? st.d_off + (uint32_t)k * (uint32_t)ld * 4u : OOB;
+      const uint32_t off = k < k_limit ? st.d_off + (uint32_t)k * (uint32_t)ld * 4u : OOB;
       reg[e] = buf_load(st.rsrc, off | (st.d_off & OOB));
     }
   }
@@ -127,9 +128,9 @@ struct PlainAlong {
 };
 
 // element(d, k) = base[d * ld + k]        (reduction contiguous in memory)
-template <int D>
+template <int D, int BK>
 struct PlainAcross {
-  using Map = AcrossMap<D>;
+  using Map = AcrossMap<D, BK>;
   static constexpr int EPT = Map::EPT;
   const float *base;
   uint32_t bytes;
@@ -149,9 +150,9 @@ struct PlainAcross {
       st.row_off[e] = d < d_extent ? (uint32_t)d * (uint32_t)ld * 4u : OOB;
     }
   }
-  __device__ inline void load(const State &st, int k0, float (&reg)[EPT]) const {
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
     const int k = k0 + st.map.k_local;
-    const uint32_t k_off = k < k_extent ? (uint32_t)k * 4u : OOB;
+    const uint32_t k_off = k < k_limit ? (uint32_t)k * 4u : OOB;
 #pragma unroll
     for (int e = 0; e < EPT; ++e) reg[e] = buf_load(st.rsrc, (st.row_off[e] + k_off) | ((st.row_off[e] | k_off) & OOB));
   }
@@ -186,7 +187,7 @@ struct StoreRowMajor {
 // workgroups that share one B tile (the large, gathered operand) also share an
 // L2.  Every wave executes the same number of barriers and exits after its
 // epilogue; there is no data-dependent loop.
-template <int BM, int BN, class ALoader, class BLoader, class Epilogue>
+template <int BM, int BN, int BK, class ALoader, class BLoader, class Epilogue>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const BLoader bl, const Epilogue ep,
                                                       int k_extent, int k_per_split, int tiles_m, int tiles_n) {
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
@@ -229,41 +230,57 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   float ra[ALoader::EPT], rb[BLoader::EPT];
-  if (k_begin < k_end) {
-    al.load(sa, k_begin, ra);
-    bl.load(sb, k_begin, rb);
-    al.template store<LDA>(sa, As[0], ra);
-    bl.template store<LDB>(sb, Bs[0], rb);
-  }
+  al.load(sa, k_begin, k_end, ra);
+  bl.load(sb, k_begin, k_end, rb);
+  al.template store<LDA>(sa, As[0], ra);
+  bl.template store<LDB>(sb, Bs[0], rb);
   __syncthreads();
 
   const int lrow = lane >> 5;   // which of the two k of an MFMA this lane feeds
   const int lcol = lane & 31;
   int buf = 0;
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-    const bool has_next = k0 + BK < k_end;
-    if (has_next) {
-      al.load(sa, k0 + BK, ra);
-      bl.load(sb, k0 + BK, rb);
-    }
+    // Fetch the next stage while this one is multiplied.  Past the end of the
+    // range every offset is out of bounds, so the last iteration's fetch costs no
+    // memory traffic and the loop body has no branch: loads, address arithmetic
+    // and MFMAs of one iteration are free to interleave.
+    al.load(sa, k0 + BK, k_end, ra);
+    bl.load(sb, k0 + BK, k_end, rb);
+    // keep the fetches ahead of the multiply: without this fence the scheduler
+    // sinks them next to their use and their latency is no longer hidden
+    __builtin_amdgcn_sched_barrier(0);
+    // MFMA operands are read from LDS one sub-step ahead of the MFMAs that use
+    // them (two register sets), so the LDS latency sits under the previous
+    // sub-step's matrix instructions.
+    float a[2][TM], b[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[0][i] = As[buf][lrow][wm * WM + 32 * i + lcol];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[0][j] = Bs[buf][lrow][wn * WN + 32 * j + lcol];
 #pragma unroll
     for (int kk = 0; kk < BK / 2; ++kk) {
-      const int krow = 2 * kk + lrow;
-      float a[TM], b[TN];
+      const int cur = kk & 1, nxt = cur ^ 1;
+      if (kk + 1 < BK / 2) {
+        const int krow = 2 * (kk + 1) + lrow;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[i] = As[buf][krow][wm * WM + 32 * i + lcol];
+        for (int i = 0; i < TM; ++i) a[nxt][i] = As[buf][krow][wm * WM + 32 * i + lcol];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) b[j] = Bs[buf][krow][wn * WN + 32 * j + lcol];
+        for (int j = 0; j < TN; ++j) b[nxt][j] = Bs[buf][krow][wn * WN + 32 * j + lcol];
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
     }
-    if (has_next) {
-      al.template store<LDA>(sa, As[buf ^ 1], ra);
-      bl.template store<LDB>(sb, Bs[buf ^ 1], rb);
+#pragma unroll
+    for (int kk = 0; kk < BK / 2 - 1; ++kk) {
+      __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);  // LDS reads of sub-step kk+1
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);  // MFMAs of sub-step kk
     }
+    __builtin_amdgcn_sched_barrier(0);
+    al.template store<LDA>(sa, As[buf ^ 1], ra);
+    bl.template store<LDB>(sb, Bs[buf ^ 1], rb);
     __syncthreads();
     buf ^= 1;
   }
@@ -287,7 +304,7 @@ struct Geometry {
   int tiles_m, tiles_n, splits, k_per_split;
   unsigned blocks() const { return (unsigned)(tiles_m * tiles_n * splits); }
 };
-inline Geometry make_geometry(int M, int N, int K, int bm, int bn, int splits) {
+inline Geometry make_geometry(int M, int N, int K, int bm, int bn, int splits, int BK = 32) {
   Geometry g;
   g.tiles_m = (M + bm - 1) / bm;
   g.tiles_n = (N + bn - 1) / bn;

@@ -87,10 +87,6 @@ struct ConvDesc {
   int K, R, S;         // filter (K output channels, C input channels)
   int P, Q;            // output spatial
   int pad_h, pad_w, u, v;
-  // device tables built lazily on first use (conv.hip); indexed by the
-  // reduction index of each implicit GEMM
-  int *fwd_tab;        // [C*R*S] x 2: element offset c*H*W + r*W + s, packed (r<<16|s)
-  int *dgrad_tab;      // [K*R*S] x 2: element offset k*P*Q - r*Q - s, packed taps
 };
 
 struct PoolDesc {

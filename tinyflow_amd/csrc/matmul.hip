@@ -28,31 +28,31 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float *__restrict_
   }
 }
 
-template <int BM, int BN, class AL, class BL>
+template <int BM, int BN, int BK, class AL, class BL>
 void launch(const AL &al, const BL &bl, const StoreRowMajor &ep, int K, const Geometry &g, hipStream_t s) {
-  hipLaunchKernelGGL((gemm_kernel<BM, BN, AL, BL, StoreRowMajor>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl,
-                     ep, K, g.k_per_split, g.tiles_m, g.tiles_n);
+  hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, StoreRowMajor>), dim3(g.blocks()), dim3(THREADS), 0, s,
+                     al, bl, ep, K, g.k_per_split, g.tiles_m, g.tiles_n);
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int BK>
 void dispatch(const float *A, bool tA, int lda, uint32_t a_bytes, const float *B, bool tB, int ldb,
               uint32_t b_bytes, const StoreRowMajor &ep, int M, int N, int K, const Geometry &g, hipStream_t s) {
   if (!tA && !tB) {
-    PlainAcross<BM> al{A, a_bytes, lda, M, K};
-    PlainAlong<BN> bl{B, b_bytes, ldb, N, K};
-    launch<BM, BN>(al, bl, ep, K, g, s);
+    PlainAcross<BM, BK> al{A, a_bytes, lda, M, K};
+    PlainAlong<BN, BK> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN, BK>(al, bl, ep, K, g, s);
   } else if (tA && !tB) {
-    PlainAlong<BM> al{A, a_bytes, lda, M, K};
-    PlainAlong<BN> bl{B, b_bytes, ldb, N, K};
-    launch<BM, BN>(al, bl, ep, K, g, s);
+    PlainAlong<BM, BK> al{A, a_bytes, lda, M, K};
+    PlainAlong<BN, BK> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN, BK>(al, bl, ep, K, g, s);
   } else if (!tA && tB) {
-    PlainAcross<BM> al{A, a_bytes, lda, M, K};
-    PlainAcross<BN> bl{B, b_bytes, ldb, N, K};
-    launch<BM, BN>(al, bl, ep, K, g, s);
+    PlainAcross<BM, BK> al{A, a_bytes, lda, M, K};
+    PlainAcross<BN, BK> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN, BK>(al, bl, ep, K, g, s);
   } else {
-    PlainAlong<BM> al{A, a_bytes, lda, M, K};
-    PlainAcross<BN> bl{B, b_bytes, ldb, N, K};
-    launch<BM, BN>(al, bl, ep, K, g, s);
+    PlainAlong<BM, BK> al{A, a_bytes, lda, M, K};
+    PlainAcross<BN, BK> bl{B, b_bytes, ldb, N, K};
+    launch<BM, BN, BK>(al, bl, ep, K, g, s);
   }
 }
 
@@ -100,10 +100,12 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   if (K == 0) return DLGpuArraySet(matC, 0.f, stream);
 
   const int lda = (int)matA->shape[1], ldb = (int)matB->shape[1];
-  const bool big = M > 64 && N > 64 && cdiv(M, 128) * cdiv(N, 128) >= num_cus();
+  bool big = M > 64 && N > 64 && cdiv(M, 128) * cdiv(N, 128) >= num_cus();
+  if (const char *e = getenv("TF_EXP_TILE")) big = atoi(e) == 128;
   const int bm = big ? 128 : 64, bn = big ? 128 : 64;
   const int tiles = cdiv(M, bm) * cdiv(N, bn);
-  const int splits = choose_splits(tiles, (int)K, 8 * BK);
+  int splits = choose_splits(tiles, (int)K, 256);
+  if (const char *e = getenv("TF_EXP_SPLITS")) splits = atoi(e);
   Geometry g = make_geometry((int)M, (int)N, (int)K, bm, bn, splits);
 
   float *dst = (float *)matC->data;
@@ -118,10 +120,10 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   }
   StoreRowMajor ep{dst, (int)N, (int)M, (int)N, M * N};
   if (big)
-    dispatch<128, 128>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
+    dispatch<128, 128, 16>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
                        transposeB, ldb, (uint32_t)b_bytes, ep, (int)M, (int)N, (int)K, g, s);
   else
-    dispatch<64, 64>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
+    dispatch<64, 64, 32>((const float *)matA->data, transposeA, lda, (uint32_t)a_bytes, (const float *)matB->data,
                      transposeB, ldb, (uint32_t)b_bytes, ep, (int)M, (int)N, (int)K, g, s);
   if (partial) {
     launch_split_sum(partial, (float *)matC->data, M * N, g.splits, s);

@@ -4,10 +4,12 @@
 // builder (src/gpu_op.cu:2839-3024).  NCHW; lanes run along the innermost (w / q)
 // index so loads and stores coalesce.
 //
-// Max-pool backward is a gather: one lane per INPUT pixel looks at the (few)
-// windows that cover it and takes dy from those whose maximum it is.  Among
-// equal maxima the first one in row-major window order wins, so the result is
-// deterministic and needs no atomics even when windows overlap (3x3 stride 2).
+// Max-pool backward runs in two passes: one lane per WINDOW records the tap that
+// holds the window's maximum (among equal maxima the first one in row-major
+// window order), then one lane per INPUT pixel gathers dy from the (few) windows
+// that cover it and name it.  A gather needs no atomics, so the result is
+// deterministic even when windows overlap (3x3 stride 2), and the forward output
+// y is not needed.
 #include "internal.h"
 
 using namespace tf;
@@ -52,9 +54,42 @@ __device__ inline int ceil_div_floor0(int a, int b) {  // ceil(a / b) clamped at
   return a <= 0 ? 0 : (a + b - 1) / b;
 }
 
+// Max-pool backward, pass 1: one lane per window records which tap (r * fw + s)
+// holds the window's first maximum in row-major order.
+__global__ __launch_bounds__(kThreads) void pool_argmax_kernel(const float *__restrict__ x,
+                                                              unsigned char *__restrict__ tap, PoolParams pp,
+                                                              int64_t total) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int q = (int)(i % pp.Q);
+    const int64_t t = i / pp.Q;
+    const int p = (int)(t % pp.P);
+    const int64_t nc = t / pp.P;
+    const float *plane = x + nc * pp.H * pp.W;
+    const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+    float best = -INFINITY;
+    int arg = 255;  // stays 255 when the window holds no comparable value (all NaN)
+    for (int r = 0; r < pp.fh; ++r) {
+      const int h = h0 + r;
+      if ((unsigned)h >= (unsigned)pp.H) continue;
+      for (int s = 0; s < pp.fw; ++s) {
+        const int w = w0 + s;
+        if ((unsigned)w >= (unsigned)pp.W) continue;
+        const float val = plane[h * pp.W + w];
+        if (val > best || (arg == 255 && val == best)) {  // strict: the first maximum wins
+          best = val;
+          arg = r * pp.fw + s;
+        }
+      }
+    }
+    tap[i] = (unsigned char)arg;
+  }
+}
+
+// Pass 2 (max) / the whole backward (mean): one lane per INPUT pixel gathers dy
+// from the windows that cover it.
 template <bool MAX>
-__global__ __launch_bounds__(kThreads) void pool_backward_kernel(const float *__restrict__ x,
-                                                                const float *__restrict__ y,
+__global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned char *__restrict__ tap,
                                                                 const float *__restrict__ dy,
                                                                 float *__restrict__ dx, PoolParams pp,
                                                                 int64_t total) {
@@ -71,38 +106,20 @@ __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const float *__
     const int q_lo = ceil_div_floor0(w + pp.pad_w - pp.fw + 1, pp.v);
     int q_hi = (w + pp.pad_w) / pp.v;
     if (q_hi > pp.Q - 1) q_hi = pp.Q - 1;
-    const float *xp = x + nc * pp.H * pp.W;
-    const float *yp = y + nc * pp.P * pp.Q;
-    const float *dyp = dy + nc * pp.P * pp.Q;
-    const float mine = MAX ? xp[h * pp.W + w] : 0.f;
+    const int64_t win_base = nc * pp.P * pp.Q;
     float acc = 0.f;
-    for (int p = p_lo; p <= p_hi; ++p)
+    for (int p = p_lo; p <= p_hi; ++p) {
+      const int r = h - (p * pp.u - pp.pad_h);
       for (int q = q_lo; q <= q_hi; ++q) {
-        if (!MAX) {
-          acc += dyp[p * pp.Q + q];
-          continue;
+        const int64_t wi = win_base + p * pp.Q + q;
+        if (MAX) {
+          const int s = w - (q * pp.v - pp.pad_w);
+          if ((int)tap[wi] == r * pp.fw + s) acc += dy[wi];
+        } else {
+          acc += dy[wi];
         }
-        if (mine != yp[p * pp.Q + q]) continue;
-        // this pixel holds the window's maximum; it receives dy unless an
-        // earlier position (row-major) of the same window holds it too
-        const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
-        bool first = true;
-        for (int r = 0; r < pp.fh && first; ++r) {
-          const int hh = h0 + r;
-          if (hh > h) break;
-          if (hh < 0) continue;
-          for (int s = 0; s < pp.fw; ++s) {
-            const int ww = w0 + s;
-            if (hh == h && ww >= w) break;
-            if ((unsigned)ww >= (unsigned)pp.W) continue;
-            if (xp[hh * pp.W + ww] == mine) {
-              first = false;
-              break;
-            }
-          }
-        }
-        if (first) acc += dyp[p * pp.Q + q];
       }
+    }
     dx[i] = MAX ? acc : acc / (float)(pp.fh * pp.fw);
   }
 }
@@ -196,13 +213,20 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
   const int64_t total = numel(dinput);
   if (total == 0) return 0;
   const PoolParams pp = params_of(d);
-  if (d->mode == 0)
-    hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s,
-                       (const float *)input->data, (const float *)output->data, (const float *)doutput->data,
-                       (float *)dinput->data, pp, total);
-  else
+  if (d->mode == 0) {
+    TF_REQUIRE(d->fh * d->fw < 255, "max-pool windows of 255 or more taps are not supported");
+    const int64_t windows = numel(doutput);
+    unsigned char *tap = (unsigned char *)device_alloc((size_t)windows);
+    TF_REQUIRE(tap, "out of device memory for %lld bytes of arg-max scratch", (long long)windows);
+    hipLaunchKernelGGL(pool_argmax_kernel, dim3(grid_for(windows)), dim3(kThreads), 0, s,
+                       (const float *)input->data, tap, pp, windows);
+    hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
+                       (const float *)doutput->data, (float *)dinput->data, pp, total);
+    device_free(tap);  // stream-ordered reuse
+  } else {
     hipLaunchKernelGGL(pool_backward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
-                       (const float *)input->data, (const float *)output->data, (const float *)doutput->data,
-                       (float *)dinput->data, pp, total);
+                       (const unsigned char *)nullptr, (const float *)doutput->data, (float *)dinput->data, pp,
+                       total);
+  }
   return finish(s, "DLGpuPooling2DBackward");
 }
