@@ -457,6 +457,53 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
   return 0;
 }
 
+extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, const int *filter_shapes,
+                                                    int *output_shapes, int dataformat, int padding,
+                                                    const int u, const int v, void ***list) {
+  TF_REQUIRE(input_shapes && filter_shapes && output_shapes && list, "null argument");
+  TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
+  TF_REQUIRE(u >= 1 && v >= 1, "strides must be positive");
+  ConvDesc *d = new ConvDesc();
+  d->magic = kMagicConv;
+  d->N = input_shapes[0];
+  d->C = input_shapes[1];
+  d->H = input_shapes[2];
+  d->W = input_shapes[3];
+  d->K = filter_shapes[0];
+  d->R = filter_shapes[2];
+  d->S = filter_shapes[3];
+  TF_REQUIRE(filter_shapes[1] == d->C, "filter expects %d input channels, input has %d", filter_shapes[1], d->C);
+  d->pad_h = padding == 1 ? d->R / 2 : 0;  // "SAME" is a symmetric k/2, "VALID" is 0
+  d->pad_w = padding == 1 ? d->S / 2 : 0;
+  d->u = u;
+  d->v = v;
+  TF_REQUIRE(d->H + 2 * d->pad_h >= d->R && d->W + 2 * d->pad_w >= d->S, "filter larger than padded input");
+  d->P = 1 + (d->H + 2 * d->pad_h - d->R) / u;
+  d->Q = 1 + (d->W + 2 * d->pad_w - d->S) / v;
+  TF_REQUIRE(d->R < 32768 && d->S < 32768, "filter extent too large");
+  d->fwd_tab = nullptr;
+  d->dgrad_tab = nullptr;
+  output_shapes[0] = d->N;
+  output_shapes[1] = d->K;
+  output_shapes[2] = d->P;
+  output_shapes[3] = d->Q;
+  // four slots like the reference's {x, w, conv, y} descriptor list
+  void **slots = (void **)malloc(sizeof(void *) * 4);
+  for (int i = 0; i < 4; ++i) slots[i] = d;
+  *list = slots;
+  return 0;
+}
+
+static int check_conv_arrays(const ConvDesc *d, const DLArray *x, const DLArray *w, const DLArray *y) {
+  TF_REQUIRE(on_gpu(x) && on_gpu(w) && on_gpu(y), "arrays must live on the GPU");
+  TF_REQUIRE(shape_is(x, d->N, d->C, d->H, d->W), "input does not match the descriptor (N,C,H,W)");
+  TF_REQUIRE(shape_is(w, d->K, d->C, d->R, d->S), "filter does not match the descriptor (K,C,R,S)");
+  TF_REQUIRE(shape_is(y, d->N, d->K, d->P, d->Q), "output does not match the descriptor (N,K,P,Q)");
+  TF_REQUIRE(numel(x) * 4 < kMaxBytes && numel(y) * 4 < kMaxBytes && numel(w) * 4 < kMaxBytes,
+             "tensors of 2 GiB or more are not supported");
+  return 0;
+}
+
 extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArrayHandle filter,
                                          DLArrayHandle output, void ***list, void **handle,
                                          int *memorytoSaving, void **stream) {
