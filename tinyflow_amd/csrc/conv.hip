@@ -480,9 +480,7 @@ extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, con
   TF_REQUIRE(d->H + 2 * d->pad_h >= d->R && d->W + 2 * d->pad_w >= d->S, "filter larger than padded input");
   d->P = 1 + (d->H + 2 * d->pad_h - d->R) / u;
   d->Q = 1 + (d->W + 2 * d->pad_w - d->S) / v;
-  TF_REQUIRE(d->R < 32768 && d->S < 32768, "filter extent too large");
-  d->fwd_tab = nullptr;
-  d->dgrad_tab = nullptr;
+  TF_REQUIRE(d->R <= 32 && d->S <= 32, "filter extents above 32 are not supported");
   output_shapes[0] = d->N;
   output_shapes[1] = d->K;
   output_shapes[2] = d->P;
