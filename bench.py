@@ -165,7 +165,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--batch", type=int, default=None, help="default: the configuration's own batch size")
+    ap.add_argument("--mem-limit-gb", type=float, default=0.0,
+                    help="cap the device allocator and run the step with the swapping executor "
+                         "(configuration 5: resnet152 at batch 128 under 16)")
     ap.add_argument("--bn-mode", default="pre_activation", choices=["pre_activation", "spatial"],
                     help="pre_activation is what every model graph of the reference passes")
     ap.add_argument("--config", default="resnet50", choices=["resnet50", "vgg16", "lenet5", "mlp", "resnet152"])
@@ -186,11 +189,19 @@ def main():
 
     hip = Hip()
     timer = ConvTimer(hip, gpu_op, _LIB)
+    if args.batch is None:
+        args.batch = {"mlp": 128, "lenet5": 64, "vgg16": 32, "resnet50": 64, "resnet152": 128}[args.config]
     kw = {"batch": args.batch}
     if args.config.startswith("resnet"):
         kw["bn_mode"] = args.bn_mode
     model, X, y = models.build(args.config, **kw)
-    ex = TrainExecutor(model.loss, 0.01)
+    if args.mem_limit_gb > 0:
+        from tinyflow_amd.SwapExecute import SwapExecutor
+        limit = int(args.mem_limit_gb * (1 << 30))
+        gpu_op.set_device_memory_limit(limit)
+        ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=int(0.85 * limit))
+    else:
+        ex = TrainExecutor(model.loss, 0.01)
     ex.init_Variable(dict(model.variables))
     feed = {model.X: X, model.y_: y}
 
@@ -198,6 +209,9 @@ def main():
         loss = ex.run(feed)[0]
     hip.sync()
 
+    swap_before = ex.swap_report() if args.mem_limit_gb > 0 else None
+    if swap_before:
+        gpu_op.device_memory_stats(reset_peak=True)
     timer.enabled = not args.no_kernel_events
     e_start, e_end = hip.event(), hip.event()
     s = stream_handle(ex.cudaStream)
@@ -246,6 +260,22 @@ def main():
         "gpu_ms_per_step": gpu_ms / args.steps, "loss": loss_val,
         "roofline": roofline,
     }
+    if swap_before:
+        after = ex.swap_report()
+        moved = {k: after[k] - swap_before[k] for k in after}
+        reserved, _, peak = gpu_op.device_memory_stats()
+        result["swap"] = {
+            "device_budget_bytes": int(args.mem_limit_gb * (1 << 30)), "peak_in_use_bytes": peak,
+            "reserved_bytes": reserved,
+            "offload_bytes_per_step": moved["offload_bytes"] / args.steps,
+            "prefetch_bytes_per_step": (moved["prefetch_bytes"] + moved["passive_bytes"]) / args.steps,
+            "offload_GBps_while_copying": moved["offload_bytes"] / max(moved["offload_seconds"], 1e-9) / 1e9,
+            "prefetch_GBps_while_copying": moved["prefetch_bytes"] / max(moved["prefetch_seconds"], 1e-9) / 1e9,
+            "pcie_GBps_over_step": (moved["offload_bytes"] + moved["prefetch_bytes"] + moved["passive_bytes"])
+                                   / wall / 1e9,
+            "passive_swap_in": moved["passive_swap_in"], "passive_swap_out": moved["passive_swap_out"],
+        }
+        ex.close()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.bn_mode, args.cpu_batch, 224, 2)
     print(json.dumps(result))

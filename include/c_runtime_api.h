@@ -72,6 +72,19 @@ int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle strea
 /* ref: c_runtime_api.h:564, gpu_op.cu:4896-4898 */
 int getInt(int *intp);
 
+/* No counterpart in the reference (which is bounded by the physical card): a
+ * device-memory budget for the allocator behind DLArrayAlloc and the ops'
+ * scratch, so that a 16 GB device can be imitated on a larger one; bytes <= 0
+ * removes it.  The environment variable TINYFLOW_GPU_MEM_LIMIT_MB sets the same
+ * budget at start-up. */
+int DLGpuSetDeviceMemoryLimit(int64_t bytes);
+
+/* No counterpart in the reference: allocator statistics in bytes -- held from
+ * HIP (in use + cached), in use, and the high-water mark of bytes in use since
+ * the last call that passed reset_peak != 0. */
+int DLGpuGetDeviceMemoryStats(int64_t *reserved, int64_t *in_use, int64_t *peak_in_use,
+                              int reset_peak);
+
 /* Pageable-vs-pinned host<->device bandwidth probe (prints GB/s).
  * ref: c_runtime_api.h:565, gpu_op.cu:4915-5005 */
 int testPcie();

@@ -1,0 +1,120 @@
+"""Swap path: activations moved to pinned host memory on a side stream and back.
+
+Checks (i) byte-exact round trips device -> pinned host -> device on a side
+stream while the compute stream is busy, (ii) that a training step executed with
+releases + swapping is bit-identical to the plain executor's step, (iii) that the
+swapping executor fits a device budget the plain executor does not fit, and that
+the budget convention of DLArrayAlloc (report the size, return no array) holds.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _shallow_resnet(batch=16, image=64, width=8):
+    from tinyflow_amd import models
+    rng = np.random.RandomState(9)
+    X, y = models.synthetic_batch(rng, (batch, 3, image, image), 10, "normal")
+    model = models.resnet(rng, [2, 1, 1, 1], batch, image=image, n_class=10, bn_mode="pre_activation", width=width)
+    return model, X, y
+
+
+def test_round_trip_on_side_stream_is_byte_exact(rt):
+    from tinyflow_amd import gpu_op, ndarray
+    side = gpu_op.create_cudaStream()
+    rng = np.random.RandomState(30)
+    arrays = [rng.normal(0, 1, s).astype(np.float32) for s in [(64, 64, 56, 56), (3, 5, 7), (1,), (1 << 20,)]]
+    busy_a = ndarray.array(rng.normal(0, 1, (2048, 2048)).astype(np.float32), rt.ctx)
+    busy_c = ndarray.empty((2048, 2048), rt.ctx)
+    for x in arrays:
+        dev = ndarray.array(x, rt.ctx)
+        for _ in range(4):   # keep the compute stream busy while the copies run
+            gpu_op.matrix_multiply(busy_a, False, busy_a, False, busy_c, rt.cublas, rt.stream)
+        host = ndarray.empty(x.shape, ndarray.cpu(0))
+        dev.copyto(host, side)
+        dev.free_gpu()
+        back = host.copyto(rt.ctx, side)
+        assert back.asnumpy().tobytes() == x.tobytes()
+    gpu_op.destroy_cudaStream(side)
+
+
+def test_pcie_probe_runs():
+    from tinyflow_amd import gpu_op
+    gpu_op.testPcie()
+
+
+def test_swapped_step_is_bit_identical_to_plain_step():
+    from tinyflow_amd.SwapExecute import SwapExecutor
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    results = []
+    for kind in ("plain", "release", "swap"):
+        model, X, y = _shallow_resnet()
+        if kind == "plain":
+            ex = TrainExecutor(model.loss, 0.01)
+        else:
+            ex = SwapExecutor(model.loss, 0.01, swap=(kind == "swap"), min_swap_bytes=1 << 12, prefetch_distance=4)
+            ex.keep_values = set(ex.Variable_node_grad_list)
+        ex.init_Variable(dict(model.variables))
+        feed = {model.X: X, model.y_: y}
+        steps = []
+        for _ in range(3):
+            out = ex.run(feed)
+            grads = [ex.value_of(g).asnumpy() for g in ex.Variable_node_grad_list]
+            steps.append(([o.asnumpy() for o in out], grads))
+        if kind == "swap":
+            rep = ex.swap_report()
+            assert rep["offload_bytes"] > 0 and rep["prefetch_bytes"] == rep["offload_bytes"]
+            assert rep["passive_swap_in"] == 0
+        if kind != "plain":
+            ex.close()
+        results.append(steps)
+    for other in results[1:]:
+        for (out_a, g_a), (out_b, g_b) in zip(results[0], other):
+            for a, b in zip(out_a + g_a, out_b + g_b):
+                assert a.tobytes() == b.tobytes()
+
+
+def test_swapping_fits_a_budget_the_plain_executor_does_not():
+    from tinyflow_amd import gpu_op, ndarray
+    from tinyflow_amd.SwapExecute import SwapExecutor
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    gpu_op.set_device_memory_limit(0)
+    peaks = {}
+    try:
+        for kind in ("plain", "release", "swap"):
+            model, X, y = _shallow_resnet(batch=32, image=96, width=16)
+            base = gpu_op.device_memory_stats(reset_peak=True)[1]
+            if kind == "plain":
+                ex = TrainExecutor(model.loss, 0.01)
+            else:
+                ex = SwapExecutor(model.loss, 0.01, swap=(kind == "swap"), min_swap_bytes=1 << 16,
+                                  prefetch_distance=4)
+            ex.init_Variable(dict(model.variables))
+            loss = None
+            for _ in range(2):
+                loss = ex.run({model.X: X, model.y_: y})[0].asnumpy()
+            peaks[kind] = (gpu_op.device_memory_stats()[2] - base, float(loss[0]))
+            if kind != "plain":
+                ex.close()
+            del ex
+        assert peaks["release"][0] < 0.7 * peaks["plain"][0]
+        assert peaks["swap"][0] < 0.9 * peaks["release"][0]
+        assert peaks["plain"][1] == peaks["release"][1] == peaks["swap"][1]
+        # a budget between the two: the swapping executor runs, a plain allocation of the rest does not
+        base = gpu_op.device_memory_stats()[1]
+        budget = base + int(peaks["swap"][0] * 1.15)
+        gpu_op.set_device_memory_limit(budget)
+        model, X, y = _shallow_resnet(batch=32, image=96, width=16)
+        ex = SwapExecutor(model.loss, 0.01, swap=True, min_swap_bytes=1 << 16, prefetch_distance=4)
+        ex.init_Variable(dict(model.variables))
+        for _ in range(2):
+            loss = ex.run({model.X: X, model.y_: y})[0].asnumpy()
+        assert float(loss[0]) == peaks["swap"][1]
+        assert gpu_op.device_memory_stats()[2] <= budget
+        ex.close()
+        # the allocation convention under the budget: an int (bytes wanted), no array
+        too_big = ndarray.empty((budget // 4 + 1024,), ndarray.gpu(0))
+        assert isinstance(too_big, int)
+    finally:
+        gpu_op.set_device_memory_limit(0)

@@ -282,3 +282,49 @@ def test_resnet50_parameter_count_at_full_width():
     finally:
         models._Builder = orig
     assert sum(int(np.prod(s)) for s in shapes) == 25503912
+
+
+# ------------------------------------------------------------- swap schedule
+
+def test_swap_schedule_orders_every_transfer_around_its_uses():
+    """plan_schedule on the LeNet training graph: every offloaded value is a
+    forward value with a backward use; it leaves after its last forward use, comes
+    back before its first backward use and is released only after its last use."""
+    from tinyflow_amd import autodiff as ad, models
+    from tinyflow_amd.SwapExecute import plan_schedule
+    from tinyflow_amd.TrainExecute import getcomputelist, swapsgd
+    rng = np.random.RandomState(0)
+    model = models.build("lenet", rng=rng) if hasattr(models, "CONFIGS") and "lenet" in models.CONFIGS \
+        else models.lenet5(rng, 8)
+    variables = ad.get_Variable_node_list(model.loss)
+    variables.reverse()
+    grads = ad.gradients(model.loss, variables)
+    topo = swapsgd(ad.find_topo_sort(getcomputelist(variables, grads, 0.1)))
+    forward = set(ad.find_topo_sort([model.loss]))
+    keep = set(variables) | {model.X, model.y_, model.loss}
+    swap_out, swap_in, release = plan_schedule(topo, forward, keep, lambda n: True, 2)
+    pos = {n: i for i, n in enumerate(topo)}
+    uses = {}
+    for n in topo:
+        for inp in n.inputs:
+            uses.setdefault(inp, []).append(pos[n])
+    out_at = {n: t for t, ns in swap_out.items() for n in ns}
+    in_at = {n: t for t, ns in swap_in.items() for n in ns}
+    rel_at = {n: t for t, ns in release.items() for n in ns}
+    assert out_at and set(out_at) == set(in_at)
+    first_backward = min(pos[n] for n in topo if n not in forward and n.isw not in (1, 2))
+    for n, t_out in out_at.items():
+        assert n in forward and n not in keep
+        fwd = [u for u in uses[n] if u < first_backward]
+        bwd = [u for u in uses[n] if u >= first_backward]
+        assert bwd, "offloaded value without a backward use"
+        assert t_out >= max(fwd + [pos[n]])
+        assert t_out < in_at[n] < bwd[0]
+        assert rel_at[n] == max(uses[n])
+    for n in keep:
+        assert n not in rel_at and n not in out_at
+    # every value that is not kept is released exactly once, never before its last use
+    for n in topo:
+        if n in keep or n.issgd:
+            continue
+        assert rel_at[n] == max(uses.get(n, [pos[n]]))

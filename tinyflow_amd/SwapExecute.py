@@ -1,0 +1,407 @@
+"""Training-step executor with activation swapping under a device-memory budget.
+
+Counterpart of the swap protocol of the reference's ``Executor`` and its
+``MemoryManager`` thread (pycode/tinyflow/autodiff.py:31-150, 2631-2836): node
+values are allocated when they are computed and released after their last use,
+forward activations that backward needs again are copied to pinned host memory on
+a side stream and dropped from the device, and copied back shortly before their
+first backward use.  The copies go through ``DLArrayCopyFromTo`` with a stream
+cell, i.e. ``hipMemcpyAsync`` on a stream of their own, ordered after the compute
+stream by events inside the library; they run on worker threads (ctypes releases
+the GIL for the duration of the call), so they overlap with kernel launches.
+
+Where the reference takes its swap / release lists from the TENSILE planner
+process, this executor derives a static vDNN-style schedule from the graph
+itself (``plan_schedule``); the lists have the reference's shape --
+``(tensor, trigger node, to_gpu)`` and ``(trigger node, tensor)``
+(pycode/tinyflow/Scheduler.py:304-331) -- so a planner could supply them instead.
+
+The device budget is enforced by the allocator behind ``DLArrayAlloc``
+(environment variable ``TINYFLOW_GPU_MEM_LIMIT_MB``, read when the library
+first allocates), not by this module.
+"""
+import queue
+import threading
+import time
+
+import numpy as np
+
+from . import autodiff as ad
+from . import gpu_op, ndarray
+from .TrainExecute import getcomputelist, swapsgd
+
+GPU, HOST, MOVING_OUT, MOVING_IN, FREED = "gpu", "host", "out", "in", "freed"
+
+
+class _Tensor(object):
+    """Where the value of one node currently lives."""
+    __slots__ = ["node", "shape", "gpu", "host", "state", "ready", "nbytes"]
+
+    def __init__(self, node, shape):
+        self.node = node
+        self.shape = shape
+        self.gpu = None
+        self.host = None
+        self.state = FREED
+        self.ready = threading.Event()
+        self.nbytes = 4 * int(np.prod(shape))
+
+
+class MemoryManager(threading.Thread):
+    """Worker that moves tensors between device and pinned host memory on its own stream."""
+
+    def __init__(self, name, ctx):
+        threading.Thread.__init__(self, name=name, daemon=True)
+        self.tasks = queue.Queue()
+        self.ctx = ctx
+        self.cpu_ctx = ndarray.cpu(0)
+        self.stream = gpu_op.create_cudaStream()
+        self.bytes_moved = 0
+        self.busy_seconds = 0.0
+        self.deferred = 0
+        self.error = None
+        self.progress = threading.Condition()
+        self.pending = 0
+
+    def submit(self, tensor, to_gpu):
+        tensor.ready.clear()
+        tensor.state = MOVING_IN if to_gpu else MOVING_OUT
+        with self.progress:
+            self.pending += 1
+        self.tasks.put((tensor, to_gpu))
+
+    def wait_for_progress(self, timeout):
+        """Block until one more queued transfer has finished (or nothing is queued)."""
+        with self.progress:
+            if self.pending:
+                self.progress.wait(timeout)
+
+    def stop(self):
+        self.tasks.put(None)
+
+    def run(self):
+        while True:
+            task = self.tasks.get()
+            if task is None:
+                return
+            tensor, to_gpu = task
+            try:
+                t0 = time.perf_counter()
+                if to_gpu:
+                    self._swap_in(tensor)
+                else:
+                    self._swap_out(tensor)
+                self.busy_seconds += time.perf_counter() - t0
+            except BaseException as e:  # surfaced by the executor thread
+                self.error = e
+            finally:
+                tensor.ready.set()
+                with self.progress:
+                    self.pending -= 1
+                    self.progress.notify_all()
+
+    def _swap_out(self, tensor):
+        if tensor.host is None:
+            host = ndarray.empty(tensor.shape, self.cpu_ctx)  # pinned, recycled by the library's pool
+            if isinstance(host, int):
+                raise MemoryError("pinned host memory exhausted (%d bytes wanted)" % host)
+            tensor.host = host
+        tensor.gpu.copyto(tensor.host, self.stream)  # returns once the copy has completed
+        gpu_arr, tensor.gpu = tensor.gpu, None
+        gpu_arr.free_gpu()
+        tensor.state = HOST
+        self.bytes_moved += tensor.nbytes
+
+    def _swap_in(self, tensor):
+        arr = None
+        for _ in range(20):  # the executor thread frees memory as it advances
+            arr = ndarray.empty(tensor.shape, self.ctx)
+            if not isinstance(arr, int):
+                break
+            time.sleep(0.002)
+        if isinstance(arr, int):
+            # no room yet: leave it on the host, the executor fetches it when it needs it
+            self.deferred += 1
+            tensor.state = HOST
+            return
+        tensor.host.copyto(arr, self.stream)
+        tensor.gpu = arr
+        tensor.state = GPU
+        self.bytes_moved += tensor.nbytes
+
+
+def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of=None, budget=None):
+    """vDNN-style static schedule.
+
+    Returns (swap_out, swap_in, release), each a dict ``trigger index -> [node]``:
+    after the node at ``trigger`` has been issued, the listed tensors are swapped
+    out / prefetched / released.  A forward value that backward uses again is
+    swapped out after its last forward use and prefetched ``prefetch_distance``
+    nodes before its first backward use; every value is released after its last
+    use.  ``keep`` (variables, feeds, the loss) is never moved or released.
+
+    With ``budget`` (bytes) and ``nbytes_of`` the schedule only moves as many
+    tensors as it takes for the simulated footprint to fit: it walks the live-bytes
+    timeline and, while its peak is above the budget, offloads the candidate that
+    spans the peak with the largest bytes x absence product (early, large
+    activations first, as vDNN does).  Without a budget every candidate moves.
+    """
+    pos = {n: i for i, n in enumerate(topo_order)}
+    uses = {}
+    for n in topo_order:
+        for inp in n.inputs:
+            uses.setdefault(inp, []).append(pos[n])
+    first_backward = min((pos[n] for n in topo_order if n not in forward_nodes and n.isw not in (1, 2)),
+                         default=len(topo_order))
+    release, last_use, candidates = {}, {}, []
+    for n in topo_order:
+        if n in keep or n.issgd:
+            continue
+        use_idx = sorted(uses.get(n, []))
+        last = use_idx[-1] if use_idx else pos[n]
+        last_use[n] = last
+        release.setdefault(last, []).append(n)
+        if n not in forward_nodes or not min_bytes_of(n):
+            continue
+        fwd_uses = [u for u in use_idx if u < first_backward]
+        bwd_uses = [u for u in use_idx if u >= first_backward]
+        if not bwd_uses:
+            continue
+        out_at = fwd_uses[-1] if fwd_uses else pos[n]
+        in_at = max(bwd_uses[0] - prefetch_distance, first_backward - 1, out_at + 1)
+        if in_at >= bwd_uses[0] or bwd_uses[0] - out_at < 2 * prefetch_distance:
+            continue  # needed again too soon for a round trip to pay
+        candidates.append((n, out_at, in_at))
+    if budget is not None:
+        candidates = _fit_budget(candidates, pos, last_use, nbytes_of, sum(nbytes_of(n) for n in keep),
+                                 budget, len(topo_order), prefetch_distance)
+    swap_out, swap_in = {}, {}
+    for n, out_at, in_at in candidates:
+        swap_out.setdefault(out_at, []).append(n)
+        swap_in.setdefault(in_at, []).append(n)
+    return swap_out, swap_in, release
+
+
+def _fit_budget(candidates, pos, last_use, nbytes_of, persistent, budget, steps, lag):
+    """Smallest greedy subset of ``candidates`` whose removal brings the simulated
+    footprint under ``budget``.  A swapped-out block is counted as resident until
+    ``lag`` nodes after its trigger (its copy has to finish first)."""
+    live = np.zeros(steps + 1, dtype=np.int64)
+    for n, born in pos.items():
+        if n in last_use:
+            live[born] += nbytes_of(n)
+            live[last_use[n] + 1] -= nbytes_of(n)
+    live = np.cumsum(live)[:steps] + persistent
+    chosen, remaining = [], list(candidates)
+    while remaining:
+        peak = int(np.argmax(live))
+        if live[peak] <= budget:
+            break
+        spanning = [c for c in remaining if c[1] + lag < peak < c[2]]
+        if not spanning:
+            break
+        best = max(spanning, key=lambda c: nbytes_of(c[0]) * (c[2] - c[1]))
+        remaining.remove(best)
+        chosen.append(best)
+        live[best[1] + lag + 1:best[2]] -= nbytes_of(best[0])
+    order = {c[0]: i for i, c in enumerate(candidates)}
+    return sorted(chosen, key=lambda c: order[c[0]])
+
+
+class SwapExecutor(object):
+    """SGD step executor that keeps the device footprint small by releasing dead
+    values and swapping forward activations to pinned host memory."""
+
+    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), swap=True, min_swap_bytes=1 << 20,
+                 prefetch_distance=8, memory_budget=None):
+        self.targetloss = targetloss
+        self.ctx = ctx
+        self.Variable_node_list = ad.get_Variable_node_list(targetloss)
+        self.Variable_node_list.reverse()
+        self.Variable_node_grad_list = ad.gradients(targetloss, self.Variable_node_list)
+        eval_nodes = getcomputelist(self.Variable_node_list, self.Variable_node_grad_list, learning_rate)
+        self.topo_order = swapsgd(ad.find_topo_sort(eval_nodes))
+        self.forward_nodes = set(ad.find_topo_sort([targetloss]))
+        self.swap = swap
+        self.min_swap_bytes = min_swap_bytes
+        self.prefetch_distance = prefetch_distance
+        self.memory_budget = memory_budget   # bytes the schedule plans for; None: move every candidate
+        self.cudaStream = gpu_op.create_cudaStream()
+        self.cudnnHandle = gpu_op.create_cudnnHandle(self.cudaStream)
+        self.cublasHandle = gpu_op.create_cublasHandle(self.cudaStream)
+        self.Variable_node_np_value = None
+        self.tensors = None
+        self.keep_values = set()   # extra nodes whose values must survive the step (for inspection)
+        self.offloader = MemoryManager("tinyflow-offload", ctx)
+        self.prefetcher = MemoryManager("tinyflow-prefetch", ctx)
+        self.offloader.start()
+        self.prefetcher.start()
+        self.stats = {}
+
+    def init_Variable(self, feed_dict):
+        self.Variable_node_np_value = feed_dict
+
+    def close(self):
+        self.offloader.stop()
+        self.prefetcher.stop()
+
+    # ------------------------------------------------------------------ set-up
+
+    def _prepare(self, feed_dict):
+        shapes = {node: tuple(np.shape(v)) for node, v in feed_dict.items()}
+        for node in self.topo_order:
+            if node not in shapes:
+                shapes[node] = tuple(node.op.infer_shape(node, [shapes[i] for i in node.inputs], self.cudnnHandle))
+        self.tensors = {node: _Tensor(node, shapes[node]) for node in self.topo_order}
+        keep = set(n for n in self.topo_order if n.isw in (1, 2)) | {self.targetloss} | self.keep_values
+        self.keep = keep
+        big = lambda n: self.swap and self.tensors[n].nbytes >= self.min_swap_bytes
+        self.swap_out_at, self.swap_in_at, self.release_at = plan_schedule(
+            self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
+            nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget)
+        pos = {n: i for i, n in enumerate(self.topo_order)}
+        self.uses = {n: [] for n in self.topo_order}
+        for n in self.topo_order:
+            for inp in n.inputs:
+                self.uses[inp].append(pos[n])
+        self.evictable = [n for n in self.topo_order
+                          if self.swap and n not in keep and not n.issgd and self.uses[n]]
+        self.cursor = 0
+
+    def _alloc(self, shape, what, protect=()):
+        """Device array of ``shape``.  When the budget is exhausted: first wait for
+        queued swap-outs (each frees its block when its copy completes), then evict
+        the resident forward value whose next use is farthest away (a passive
+        swap-out, pycode/tinyflow/autodiff.py:2741-2766 in the reference)."""
+        deadline = time.perf_counter() + 120.0
+        while True:
+            arr = ndarray.empty(shape, self.ctx)
+            if not isinstance(arr, int):
+                return arr
+            self._check_workers()
+            if time.perf_counter() > deadline:
+                break
+            if self.offloader.pending or self.prefetcher.pending:
+                self.offloader.wait_for_progress(0.05)
+                continue
+            victim = self._pick_victim(protect)
+            if victim is None:
+                break
+            self.stats["passive_swap_out"] = self.stats.get("passive_swap_out", 0) + 1
+            self.offloader.submit(victim, False)
+        raise MemoryError("device budget exhausted allocating %s for %s" % (shape, what))
+
+    def _pick_victim(self, protect):
+        best, best_next = None, -1
+        for node in self.evictable:
+            t = self.tensors[node]
+            if t.state != GPU or node in protect:
+                continue
+            nxt = next((u for u in self.uses[node] if u >= self.cursor), None)
+            if nxt is None or nxt == self.cursor:
+                continue
+            if nxt > best_next:
+                best, best_next = t, nxt
+        return best
+
+    def _check_workers(self):
+        for w in (self.offloader, self.prefetcher):
+            if w.error is not None:
+                raise w.error
+
+    def _on_gpu(self, tensor, protect=()):
+        """Device array of a tensor, fetching it back first if it was swapped out."""
+        if tensor.state in (MOVING_OUT, MOVING_IN):
+            tensor.ready.wait()
+            self._check_workers()
+        if tensor.state == HOST:   # not prefetched in time: passive swap-in on the compute stream
+            self.stats["passive_swap_in"] = self.stats.get("passive_swap_in", 0) + 1
+            arr = self._alloc(tensor.shape, tensor.node.name, protect)
+            tensor.host.copyto(arr, self.cudaStream)
+            tensor.gpu, tensor.state = arr, GPU
+            self.stats["passive_bytes"] = self.stats.get("passive_bytes", 0) + tensor.nbytes
+        assert tensor.state == GPU, "%s is %s" % (tensor.node.name, tensor.state)
+        return tensor.gpu
+
+    # --------------------------------------------------------------------- step
+
+    def run(self, feed_dict, convert_to_numpy_ret_vals=False):
+        """One step; returns [loss, variables in network order]."""
+        if self.tensors is None:
+            first = dict(feed_dict)
+            first.update(self.Variable_node_np_value or {})
+            self._prepare(first)
+            feed_dict = first
+        for node, value in feed_dict.items():
+            t = self.tensors[node]
+            if node.isw == 1 and t.state == GPU:
+                continue   # variables stay on the device between steps
+            if t.gpu is None:
+                t.gpu = ndarray.array(value, ctx=self.ctx)
+                if isinstance(t.gpu, int):
+                    raise MemoryError("device budget exhausted feeding %s" % node.name)
+                t.state = GPU
+            else:
+                t.gpu._sync_copyfrom(value)
+        handles = (self.cudnnHandle, self.cublasHandle, self.cudaStream)
+        for idx, node in enumerate(self.topo_order):
+            t = self.tensors[node]
+            if node.isw in (1, 2):
+                pass
+            else:
+                self.cursor = idx
+                input_vals = [self._on_gpu(self.tensors[i], node.inputs) for i in node.inputs]
+                out = None
+                if not node.issgd:
+                    out = self._alloc(t.shape, node.name, node.inputs)
+                wanted = node.op.compute(node, input_vals, out, *handles)
+                for _ in range(3):
+                    if not wanted:
+                        break
+                    # the op found no room for its scratch: make room, hand the block
+                    # back to the allocator's cache and run the op again
+                    self._alloc(((int(wanted) + 3) // 4,), node.name + " scratch", node.inputs).free_gpu()
+                    wanted = node.op.compute(node, input_vals, out, *handles)
+                if wanted:
+                    raise MemoryError("%s: %d bytes of device scratch could not be allocated" % (node.name, wanted))
+                if out is not None:
+                    t.gpu, t.state = out, GPU
+            for n in self.swap_out_at.get(idx, ()):
+                self.offloader.submit(self.tensors[n], False)
+            for n in self.swap_in_at.get(idx, ()):
+                tn = self.tensors[n]
+                if tn.state == MOVING_OUT:
+                    tn.ready.wait()
+                if tn.state == HOST:
+                    self.prefetcher.submit(tn, True)
+            for n in self.release_at.get(idx, ()):
+                self._release(self.tensors[n])
+        self._check_workers()
+        result = [self._on_gpu(self.tensors[self.targetloss])]
+        result += [self.tensors[v].gpu for v in reversed(self.Variable_node_list)]
+        if convert_to_numpy_ret_vals:
+            return [r.asnumpy() for r in result]
+        return result
+
+    def _release(self, tensor):
+        if tensor.state in (MOVING_OUT, MOVING_IN):
+            tensor.ready.wait()
+        if tensor.gpu is not None:
+            # stream-ordered: kernels already enqueued keep reading the block safely,
+            # and whoever receives it next is enqueued behind them
+            gpu_arr, tensor.gpu = tensor.gpu, None
+            gpu_arr.free_gpu()
+        tensor.state = FREED
+
+    def value_of(self, node):
+        """Device array holding ``node`` after a step (list the node in ``keep_values`` first)."""
+        return self._on_gpu(self.tensors[node])
+
+    def swap_report(self):
+        """Bytes moved and busy time of the two copy workers since construction."""
+        return {"offload_bytes": self.offloader.bytes_moved, "offload_seconds": self.offloader.busy_seconds,
+                "prefetch_bytes": self.prefetcher.bytes_moved, "prefetch_seconds": self.prefetcher.busy_seconds,
+                "passive_swap_in": self.stats.get("passive_swap_in", 0),
+                "passive_swap_out": self.stats.get("passive_swap_out", 0),
+                "passive_bytes": self.stats.get("passive_bytes", 0),
+                "prefetch_deferred": self.prefetcher.deferred}

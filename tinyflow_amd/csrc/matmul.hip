@@ -100,12 +100,10 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   if (K == 0) return DLGpuArraySet(matC, 0.f, stream);
 
   const int lda = (int)matA->shape[1], ldb = (int)matB->shape[1];
-  bool big = M > 64 && N > 64 && cdiv(M, 128) * cdiv(N, 128) >= num_cus();
-  if (const char *e = getenv("TF_EXP_TILE")) big = atoi(e) == 128;
+  const bool big = M > 64 && N > 64 && cdiv(M, 128) * cdiv(N, 128) >= num_cus();
   const int bm = big ? 128 : 64, bn = big ? 128 : 64;
   const int tiles = cdiv(M, bm) * cdiv(N, bn);
-  int splits = choose_splits(tiles, (int)K, 256);
-  if (const char *e = getenv("TF_EXP_SPLITS")) splits = atoi(e);
+  const int splits = choose_splits(tiles, (int)K, 256);
   Geometry g = make_geometry((int)M, (int)N, (int)K, bm, bn, splits);
 
   float *dst = (float *)matC->data;

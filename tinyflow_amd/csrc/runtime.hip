@@ -21,7 +21,8 @@ namespace {
 
 struct StreamRec {
   hipStream_t stream;
-  hipEvent_t event;  // reusable marker for cross-stream ordering
+  hipEvent_t event;   // reusable marker for cross-stream ordering
+  bool runs_kernels;  // an op entry point has launched on it (copy-only streams stay false)
 };
 
 struct Runtime {
@@ -31,6 +32,8 @@ struct Runtime {
     std::multimap<size_t, void *> free_blocks;      // size -> block
     std::unordered_map<void *, size_t> block_size;  // every block obtained from HIP
     size_t reserved = 0;                            // bytes held from HIP (in use + cached)
+    size_t in_use = 0;                              // bytes handed out and not yet returned
+    size_t peak_in_use = 0;
   };
   Pool dev, host;
   size_t dev_limit = 0;  // 0 = unlimited; TINYFLOW_GPU_MEM_LIMIT_MB
@@ -58,43 +61,50 @@ size_t round_size(size_t bytes) {
   return (bytes + q - 1) / q * q;
 }
 
-// Give every cached block of `p` back to HIP.  hipFree waits for the device, so
+// Give cached blocks of `p` back to HIP, largest first, until `need` more bytes fit
+// under `limit` (everything when limit == 0).  hipFree waits for the device, so
 // blocks still referenced by enqueued kernels are safe to release.
-void release_cached(Runtime::Pool &p, bool device) {
-  for (auto &kv : p.free_blocks) {
-    if (device) (void)hipFree(kv.second); else (void)hipHostFree(kv.second);
-    p.reserved -= kv.first;
-    p.block_size.erase(kv.second);
+void release_cached(Runtime::Pool &p, bool device, size_t need, size_t limit) {
+  while (!p.free_blocks.empty()) {
+    if (limit != 0 && p.reserved + need <= limit) break;
+    auto it = std::prev(p.free_blocks.end());
+    if (device) (void)hipFree(it->second); else (void)hipHostFree(it->second);
+    p.reserved -= it->first;
+    p.block_size.erase(it->second);
+    p.free_blocks.erase(it);
   }
-  p.free_blocks.clear();
 }
 
 void *pool_alloc(Runtime::Pool &p, size_t bytes, bool device, size_t limit) {
   const size_t want = round_size(bytes);
+  void *ptr = nullptr;
   auto it = p.free_blocks.lower_bound(want);
   // accept a cached block when it wastes at most 1/8 of its size
   if (it != p.free_blocks.end() && it->first - want <= it->first / 8) {
-    void *ptr = it->second;
+    ptr = it->second;
     p.free_blocks.erase(it);
-    return ptr;
   }
-  for (int attempt = 0; attempt < 2; ++attempt) {
+  for (int attempt = 0; !ptr && attempt < 2; ++attempt) {
     if (limit == 0 || p.reserved + want <= limit) {
-      void *ptr = nullptr;
       hipError_t e = device ? hipMalloc(&ptr, want) : hipHostMalloc(&ptr, want, hipHostMallocDefault);
       if (e == hipSuccess && ptr) {
         p.block_size[ptr] = want;
         p.reserved += want;
-        return ptr;
+        break;
       }
+      ptr = nullptr;
       (void)hipGetLastError();  // clear the sticky out-of-memory error
     }
     if (attempt == 0) {
       if (p.free_blocks.empty()) break;
-      release_cached(p, device);
+      release_cached(p, device, want, limit);
     }
   }
-  return nullptr;
+  if (ptr) {
+    p.in_use += p.block_size[ptr];
+    if (p.in_use > p.peak_in_use) p.peak_in_use = p.in_use;
+  }
+  return ptr;
 }
 
 void pool_free(Runtime::Pool &p, void *ptr) {
@@ -102,6 +112,7 @@ void pool_free(Runtime::Pool &p, void *ptr) {
   auto it = p.block_size.find(ptr);
   if (it == p.block_size.end()) return;  // not ours (e.g. a borrowed numpy buffer)
   p.free_blocks.emplace(it->second, ptr);
+  p.in_use -= it->second;
 }
 
 }  // namespace
@@ -129,7 +140,20 @@ void pinned_free(void *p) {
   pool_free(r.host, p);
 }
 
-hipStream_t stream_of(void **cell) { return cell ? reinterpret_cast<hipStream_t>(*cell) : nullptr; }
+// Stream an op launches on.  Marks the stream as one that runs kernels, so that
+// copies on other streams know to order themselves behind it.
+hipStream_t stream_of(void **cell) {
+  if (!cell) return nullptr;
+  hipStream_t s = reinterpret_cast<hipStream_t>(*cell);
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  for (auto &rec : r.streams)
+    if (rec.stream == s) {
+      rec.runs_kernels = true;
+      break;
+    }
+  return s;
+}
 
 bool sync_every_op() {
   Runtime &r = rt();
@@ -232,13 +256,16 @@ hipMemcpyKind copy_kind(const DLArray *from, const DLArray *to) {
   return hipMemcpyHostToHost;
 }
 
-// Make `s` wait for everything already enqueued on the other streams created
-// through DLGpuCreatecudaStream.
+// Make `s` wait for everything already enqueued on the other kernel-running
+// streams created through DLGpuCreatecudaStream: whatever produced the source, or
+// still reads the destination's recycled storage, was launched on one of them.
+// Copy-only streams are skipped, so an offload and a prefetch stream stay
+// independent of each other.
 int wait_for_other_streams(hipStream_t s) {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
   for (auto &rec : r.streams) {
-    if (rec.stream == s) continue;
+    if (rec.stream == s || !rec.runs_kernels) continue;
     TF_HIP(hipEventRecord(rec.event, rec.stream));
     TF_HIP(hipStreamWaitEvent(s, rec.event, 0));
   }
@@ -265,7 +292,7 @@ extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamH
     if (kind == hipMemcpyDeviceToDevice) TF_HIP(hipDeviceSynchronize());
     return 0;
   }
-  hipStream_t s = stream_of(reinterpret_cast<void **>(stream));
+  hipStream_t s = reinterpret_cast<hipStream_t>(*reinterpret_cast<void **>(stream));
   if (wait_for_other_streams(s) != 0) return -1;
   TF_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, s));
   // Host memory must be readable / reusable on return.  A device-to-device copy
@@ -275,6 +302,31 @@ extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamH
 }
 
 extern "C" int getInt(int *intp) { return intp ? *intp : 0; }
+
+// Device-memory budget of the allocator (no counterpart in the reference, which
+// is bounded by the physical card): bytes <= 0 removes the limit.  Cached blocks
+// are given back until the budget holds; arrays in use are not touched.
+extern "C" int DLGpuSetDeviceMemoryLimit(int64_t bytes) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  r.init();
+  r.dev_limit = bytes > 0 ? (size_t)bytes : 0;
+  if (r.dev_limit) release_cached(r.dev, true, 0, r.dev_limit);
+  return 0;
+}
+
+// Bytes held from HIP (in use + cached), bytes in use, and the high-water mark of
+// bytes in use since the last call with reset_peak != 0 (no reference counterpart).
+extern "C" int DLGpuGetDeviceMemoryStats(int64_t *reserved, int64_t *in_use, int64_t *peak_in_use,
+                                         int reset_peak) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  if (reserved) *reserved = (int64_t)r.dev.reserved;
+  if (in_use) *in_use = (int64_t)r.dev.in_use;
+  if (peak_in_use) *peak_in_use = (int64_t)r.dev.peak_in_use;
+  if (reset_peak) r.dev.peak_in_use = r.dev.in_use;
+  return 0;
+}
 
 // ----------------------------------------------------- streams and handles
 
@@ -291,7 +343,7 @@ extern "C" int DLGpuCreatecudaStream(void **cell) {
     Runtime &r = rt();
     std::lock_guard<std::mutex> g(r.mu);
     r.init();
-    r.streams.push_back({s, ev});
+    r.streams.push_back({s, ev, false});
   }
   *cell = s;
   return 0;

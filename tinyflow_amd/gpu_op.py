@@ -376,3 +376,19 @@ def getInt(intp):
 
 def testPcie():
     check_call(_LIB.testPcie())
+
+
+# --------------------------------------------------- allocator budget (extension)
+
+def set_device_memory_limit(nbytes):
+    """Budget of the device allocator in bytes (0 or None: unlimited).  No
+    counterpart in the reference; lets a 16 GB card be imitated on a larger one."""
+    check_call(_LIB.DLGpuSetDeviceMemoryLimit(ctypes.c_int64(int(nbytes or 0))))
+
+
+def device_memory_stats(reset_peak=False):
+    """(reserved, in_use, peak_in_use) bytes of the device allocator."""
+    vals = [ctypes.c_int64(0) for _ in range(3)]
+    check_call(_LIB.DLGpuGetDeviceMemoryStats(ctypes.byref(vals[0]), ctypes.byref(vals[1]),
+                                              ctypes.byref(vals[2]), int(bool(reset_peak))))
+    return tuple(v.value for v in vals)
