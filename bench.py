@@ -66,9 +66,39 @@ def stream_handle(stream_cell):
     return ctypes.cast(stream_cell, ctypes.POINTER(ctypes.c_void_p))[0]
 
 
+# HBM bytes per launch (reads + writes) of each convolution kernel symbol in the
+# default workload, averaged over that symbol's launches in one step: rocprofv3
+# FETCH_SIZE and WRITE_SIZE counter runs of this script, scaled by what the same
+# counters read for a 256 MiB copy (x2.000 and x1.000).  The figures and the
+# commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
+# --config resnet50 --batch 64 only and are reported as null otherwise.
+MEASURED_TRAFFIC_BYTES = {
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 130996171,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 144753893,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 125048656,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 243276706,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 148761548,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 129453474,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 73266144,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreScatter>": 228940858,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 85096019,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 155676455,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 67395057,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 80470416,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 80089923,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreScatter>": 126753834,
+    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 64556296,
+    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 1>, StoreNCHW>": 60179698,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 1>, StoreNCHW>": 58760311,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 58352916,
+}
+
+
 class ConvTimer(object):
-    """Records a HIP event pair on the compute stream around every convolution
-    launch and attributes the time to the kernel variant the library reports."""
+    """Has the library record a HIP event pair on the compute stream around the
+    contraction kernel of every convolution call (the kernel alone, without the
+    layout / split-sum passes next to it) and attributes the time to the kernel
+    symbol the library reports for that call."""
 
     def __init__(self, hip, gpu_op, lib):
         self.hip, self.gpu_op, self.lib = hip, gpu_op, lib
@@ -91,12 +121,8 @@ class ConvTimer(object):
             rc = self.lib.DLGpuConvolutionDescribeKernel(cudnnlist, which, buf, 256, ctypes.byref(flops))
             if rc != 0:
                 raise RuntimeError("DLGpuConvolutionDescribeKernel failed")
-            # group by kernel symbol; calls whose reduction is split also run the
-            # small partial-sum kernel inside the bracketed region, so they are
-            # kept apart from the single-kernel calls
             variant, symbol = buf.value.decode().split(" | ")
-            split = not variant.endswith(" s1")
-            hit = ((symbol + " + split_sum_kernel") if split else symbol, flops.value)
+            hit = (symbol, flops.value)
             self._describe_cache[key] = hit
         return hit
 
@@ -112,10 +138,13 @@ class ConvTimer(object):
             variant, flops = self._describe(cudnnlist, which)
             s = stream_handle(stream)
             e0, e1 = self._event(), self._event()
-            self.hip.record(e0, s)
+            self.lib.DLGpuConvolutionTimeNextKernel(e0, e1)
             ret = fn(*args)
-            self.hip.record(e1, s)
-            self.pairs.append((variant, flops, e0, e1))
+            if ret:   # no room for scratch: nothing was launched, the caller makes room and calls again
+                self.lib.DLGpuConvolutionTimeNextKernel(None, None)
+                self.pool += [e0, e1]
+            else:
+                self.pairs.append((variant, flops, e0, e1))
             return ret
         return timed
 
@@ -177,6 +206,9 @@ def main():
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="do not record per-convolution HIP events in the timed region")
     ap.add_argument("--breakdown", action="store_true", help="print per-variant conv times to stderr")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region launch a plain copy kernel (256 MiB read, 256 MiB written, "
+                         "three times) so a counter run holds a dispatch of known traffic to scale by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)\n"
@@ -205,8 +237,12 @@ def main():
     ex.init_Variable(dict(model.variables))
     feed = {model.X: X, model.y_: y}
 
-    for _ in range(max(args.warmup, 1)):
-        loss = ex.run(feed)[0]
+    # The first run uploads the batch; later runs are given no feed, so the timed
+    # region starts with images and labels resident in device memory.
+    loss = ex.run(feed)[0]
+    resident = {}
+    for _ in range(max(args.warmup, 1) - 1):
+        loss = ex.run(resident)[0]
     hip.sync()
 
     swap_before = ex.swap_report() if args.mem_limit_gb > 0 else None
@@ -219,13 +255,33 @@ def main():
     t0 = time.perf_counter()
     hip.record(e_start, s)
     for _ in range(args.steps):
-        loss = ex.run(feed)[0]
+        loss = ex.run(resident)[0]
     hip.record(e_end, s)
     hip.sync()
     wall = time.perf_counter() - t0
     timer.enabled = False
     gpu_ms = hip.elapsed_ms(e_start, e_end)
     loss_val = float(loss.asnumpy()[0])
+    swap_after = ex.swap_report() if swap_before else None
+    swap_mem = gpu_op.device_memory_stats() if swap_before else None
+
+    # Same step with the batch handed over as host (numpy) buffers every step, as a
+    # data loader would: includes the PCIe upload.  Reported beside `value`, never as it.
+    host_steps = max(2, min(args.steps, 5))
+    hip.sync()
+    t1 = time.perf_counter()
+    for _ in range(host_steps):
+        ex.run(feed)
+    hip.sync()
+    host_fed_ms = (time.perf_counter() - t1) * 1e3 / host_steps
+
+    if args.copy_calibration:
+        from tinyflow_amd import ndarray
+        src = ndarray.array(np.ones((64 << 20,), dtype=np.float32), ndarray.gpu(0))
+        dst = ndarray.empty((64 << 20,), ndarray.gpu(0))
+        for _ in range(3):
+            gpu_op.matrix_elementwise_multiply_by_const(src, 1.0, dst, ex.cudaStream)
+        hip.sync()
 
     ms_per_step = wall * 1e3 / args.steps
     imgs_per_sec = args.batch * args.steps / wall
@@ -238,7 +294,10 @@ def main():
         achieved = total_flops / (total_ms * 1e-3) / 1e12
         roofline = {
             "bound": "mfma", "kernel": name, "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
+            "traffic": (MEASURED_TRAFFIC_BYTES.get(name) if (args.config, args.batch, args.bn_mode) ==
+                        ("resnet50", 64, "pre_activation") and not args.mem_limit_gb else None),
+            "flops_per_launch": total_flops / launches,
             "launches": launches, "avg_launch_ms": total_ms / launches,
             "share_of_step": total_ms / args.steps / (gpu_ms / args.steps),
         }
@@ -258,12 +317,13 @@ def main():
                                "softmax-xent over %d random one-hot classes, He-normal weights"
                                % (args.config, args.batch, args.bn_mode, model.n_class)},
         "gpu_ms_per_step": gpu_ms / args.steps, "loss": loss_val,
+        "host_fed": {"ms_per_step": host_fed_ms, "imgs_per_sec": args.batch * 1e3 / host_fed_ms, "steps": host_steps,
+                     "note": "batch re-uploaded from pageable host memory every step (PCIe-inclusive)"},
         "roofline": roofline,
     }
     if swap_before:
-        after = ex.swap_report()
-        moved = {k: after[k] - swap_before[k] for k in after}
-        reserved, _, peak = gpu_op.device_memory_stats()
+        moved = {k: swap_after[k] - swap_before[k] for k in swap_after}
+        reserved, _, peak = swap_mem
         result["swap"] = {
             "device_budget_bytes": int(args.mem_limit_gb * (1 << 30)), "peak_in_use_bytes": peak,
             "reserved_bytes": reserved,

@@ -215,6 +215,13 @@ int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLArrayHandle 
 int DLGpuConvolutionDescribeKernel(void ***list, int which, char *name, int name_len,
                                    double *flops);
 
+/* No counterpart in the reference: measurement aid.  The next convolution entry
+ * point called on this host thread records the two HIP events (hipEvent_t, either
+ * may be NULL) on its stream immediately before and after its contraction kernel,
+ * leaving out the layout and split-sum passes that may accompany it, so a caller
+ * can time exactly the kernel a profiler lists under the described symbol. */
+int DLGpuConvolutionTimeNextKernel(void *start_event, void *stop_event);
+
 /* ----------------------------------------------------------------- pooling */
 
 /* out = 1 + (in + 2*pad - window) / stride.

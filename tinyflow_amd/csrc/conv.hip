@@ -339,10 +339,17 @@ void pick_tile(int M, int N, int &bm, int &bn) {
   }
 }
 
+// Events a measuring caller wants recorded around the next contraction kernel only
+// (not around the layout or split-sum passes that may accompany it).
+thread_local hipEvent_t next_kernel_start = nullptr, next_kernel_stop = nullptr;
+
 template <int BM, int BN, int BK, class AL, class BL, class EP>
 void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s) {
+  if (next_kernel_start) hipEventRecord(next_kernel_start, s);
   hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl, ep,
                      K, g.k_per_split, g.tiles_m, g.tiles_n);
+  if (next_kernel_stop) hipEventRecord(next_kernel_stop, s);
+  next_kernel_start = next_kernel_stop = nullptr;
 }
 
 bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
@@ -454,6 +461,12 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
            p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, p.b_loader, p.bn, bk, p.b_mode, p.epilogue);
   if (flops)
     *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
+  return 0;
+}
+
+extern "C" int DLGpuConvolutionTimeNextKernel(void *start_event, void *stop_event) {
+  next_kernel_start = (hipEvent_t)start_event;
+  next_kernel_stop = (hipEvent_t)stop_event;
   return 0;
 }
 
