@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   if (l >= L) return;
   float v[NREG];
 #pragma unroll
-  for (int n = 0; n < NREG; ++n) v[n] = n < N ? x[(int64_t)n * L + l] : 0.f;
+  for (int n = 0; n < NREG; ++n) v[n] = n < N ? __builtin_nontemporal_load(x + (int64_t)n * L + l) : 0.f;
   float s = 0.f;
 #pragma unroll
   for (int n = 0; n < NREG; ++n) s += v[n];
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   save_istd[l] = istd;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) y[(int64_t)n * L + l] = (v[n] - mean) * istd;
+    if (n < N) __builtin_nontemporal_store((v[n] - mean) * istd, y + (int64_t)n * L + l);
 }
 
 // any N: three sweeps over the column (the second and third hit the cache)
@@ -93,8 +93,8 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
   float xh[NREG], g[NREG];
 #pragma unroll
   for (int n = 0; n < NREG; ++n) {
-    xh[n] = n < N ? x[(int64_t)n * L + l] : mean;
-    g[n] = n < N ? dy[(int64_t)n * L + l] : 0.f;
+    xh[n] = n < N ? __builtin_nontemporal_load(x + (int64_t)n * L + l) : mean;
+    g[n] = n < N ? __builtin_nontemporal_load(dy + (int64_t)n * L + l) : 0.f;
   }
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
   const float scale = istd / m;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) dx[(int64_t)n * L + l] = scale * (m * g[n] - s1 - xh[n] * s2);
+    if (n < N) __builtin_nontemporal_store(scale * (m * g[n] - s1 - xh[n] * s2), dx + (int64_t)n * L + l);
 }
 
 __global__ __launch_bounds__(kThreads) void bn_pa_backward_stream_kernel(const float *__restrict__ x,

@@ -345,10 +345,10 @@ thread_local hipEvent_t next_kernel_start = nullptr, next_kernel_stop = nullptr;
 
 template <int BM, int BN, int BK, class AL, class BL, class EP>
 void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s) {
-  if (next_kernel_start) hipEventRecord(next_kernel_start, s);
+  if (next_kernel_start) (void)hipEventRecord(next_kernel_start, s);
   hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl, ep,
                      K, g.k_per_split, g.tiles_m, g.tiles_n);
-  if (next_kernel_stop) hipEventRecord(next_kernel_stop, s);
+  if (next_kernel_stop) (void)hipEventRecord(next_kernel_stop, s);
   next_kernel_start = next_kernel_stop = nullptr;
 }
 
