@@ -28,6 +28,46 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float *__restrict_
   }
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Same sum for 16-byte aligned data with count % 4 == 0, with the splits dealt
+// round-robin to SG lane groups of a workgroup so that a small output with
+// many splits still has enough loads in flight.  Group g adds splits g, g+SG,
+// ... in that order, then group 0 adds the SG group sums in index order: the
+// order of additions depends on (splits, SG) only, never on timing.
+template <int SG>
+__global__ __launch_bounds__(256) void split_sum_vec_kernel(const f32x4 *__restrict__ partial,
+                                                           f32x4 *__restrict__ out, int64_t count4, int splits) {
+  constexpr int COLS = 256 / SG;
+  __shared__ f32x4 part[SG][COLS];
+  const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+  const int64_t i = (int64_t)blockIdx.x * COLS + col;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (i < count4) {
+    int k = g;
+    for (; k + 3 * SG < splits; k += 4 * SG) {
+      const f32x4 v0 = __builtin_nontemporal_load(partial + (int64_t)k * count4 + i);
+      const f32x4 v1 = __builtin_nontemporal_load(partial + (int64_t)(k + SG) * count4 + i);
+      const f32x4 v2 = __builtin_nontemporal_load(partial + (int64_t)(k + 2 * SG) * count4 + i);
+      const f32x4 v3 = __builtin_nontemporal_load(partial + (int64_t)(k + 3 * SG) * count4 + i);
+      acc = (((acc + v0) + v1) + v2) + v3;
+    }
+    for (; k < splits; k += SG) acc += __builtin_nontemporal_load(partial + (int64_t)k * count4 + i);
+  }
+  if (SG == 1) {
+    if (i < count4) out[i] = acc;
+    return;
+  }
+  part[g][col] = acc;
+  __syncthreads();
+  if (g == 0 && i < count4) {
+    f32x4 total = part[0][col];
+#pragma unroll
+    for (int j = 1; j < SG; ++j) total += part[j][col];
+    out[i] = total;
+  }
+}
+
 template <int BM, int BN, int BK, class AL, class BL>
 void launch(const AL &al, const BL &bl, const StoreRowMajor &ep, int K, const Geometry &g, hipStream_t s) {
   hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, StoreRowMajor>), dim3(g.blocks()), dim3(THREADS), 0, s,
@@ -61,6 +101,21 @@ void dispatch(const float *A, bool tA, int lda, uint32_t a_bytes, const float *B
 namespace tf {
 
 int launch_split_sum(const float *partial, float *out, int64_t count, int splits, hipStream_t s) {
+  const bool vec = count % 4 == 0 && ((reinterpret_cast<uintptr_t>(partial) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  if (vec) {
+    const int64_t count4 = count / 4;
+    const f32x4 *p4 = reinterpret_cast<const f32x4 *>(partial);
+    f32x4 *o4 = reinterpret_cast<f32x4 *>(out);
+    // enough lane groups that about 64 K lanes are busy, as long as each group
+    // still has a few splits to add
+    int sg = 1;
+    while (sg < 16 && count4 * sg < 65536 && splits >= 8 * sg) sg *= 4;
+    const unsigned blocks = (unsigned)((count4 + 256 / sg - 1) / (256 / sg));
+    if (sg == 1) hipLaunchKernelGGL(split_sum_vec_kernel<1>, dim3(blocks), dim3(256), 0, s, p4, o4, count4, splits);
+    else if (sg == 4) hipLaunchKernelGGL(split_sum_vec_kernel<4>, dim3(blocks), dim3(256), 0, s, p4, o4, count4, splits);
+    else hipLaunchKernelGGL(split_sum_vec_kernel<16>, dim3(blocks), dim3(256), 0, s, p4, o4, count4, splits);
+    return 0;
+  }
   int64_t blocks = (count + 255) / 256;
   const int64_t cap = (int64_t)num_cus() * 8;
   if (blocks > cap) blocks = cap;
