@@ -118,3 +118,49 @@ def test_swapping_fits_a_budget_the_plain_executor_does_not():
         assert isinstance(too_big, int)
     finally:
         gpu_op.set_device_memory_limit(0)
+
+
+def test_budget_arena_never_overlaps_and_coalesces():
+    """Random allocate / free traffic under a budget: live arrays never overlap,
+    their contents survive their neighbours' churn, and once everything is freed
+    one array of nearly the whole budget fits again (free ranges were merged)."""
+    import ctypes
+    from tinyflow_amd import gpu_op, ndarray
+    ctx = ndarray.gpu(0)
+    base = gpu_op.device_memory_stats()[1]
+    budget = 64 << 20
+    gpu_op.set_device_memory_limit(base + budget)
+    try:
+        rng = np.random.RandomState(5)
+        live = {}
+        refused = 0
+        for step in range(400):
+            if live and (rng.rand() < 0.45 or len(live) > 40):
+                key = list(live)[rng.randint(len(live))]
+                arr, value = live.pop(key)
+                assert np.all(arr.asnumpy() == value)
+                arr.free_gpu()
+            else:
+                n = int(rng.choice([64, 1000, 4096, 70000, 300000, 1 << 20, 3 << 20]))
+                arr = ndarray.empty((n,), ctx)
+                if isinstance(arr, int):
+                    refused += 1
+                    assert arr == 4 * n
+                    continue
+                value = np.float32(step)
+                gpu_op.array_set(arr, float(value), None)
+                live[step] = (arr, value)
+            spans = sorted((ctypes.cast(a.handle.contents.data, ctypes.c_void_p).value, 4 * a.shape[0])
+                           for a, _ in live.values())
+            for (p0, l0), (p1, _) in zip(spans, spans[1:]):
+                assert p0 + l0 <= p1
+            assert gpu_op.device_memory_stats()[1] - base <= budget
+        for arr, value in live.values():
+            assert np.all(arr.asnumpy() == value)
+            arr.free_gpu()
+        assert gpu_op.device_memory_stats()[1] == base
+        whole = ndarray.empty(((budget - (1 << 20)) // 4,), ctx)
+        assert not isinstance(whole, int)
+        whole.free_gpu()
+    finally:
+        gpu_op.set_device_memory_limit(0)

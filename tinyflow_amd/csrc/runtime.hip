@@ -37,6 +37,20 @@ struct Runtime {
   };
   Pool dev, host;
   size_t dev_limit = 0;  // 0 = unlimited; TINYFLOW_GPU_MEM_LIMIT_MB
+
+  // Under a budget, device memory comes from one arena obtained with a single
+  // hipMalloc and sub-allocated best-fit with coalescing: a step that runs at the
+  // budget then never calls hipMalloc / hipFree (hipFree waits for the whole
+  // device, which would stall the copy streams of the swap path on every
+  // allocation).  Blocks handed out before the budget was set stay with `dev`.
+  struct Arena {
+    char *base = nullptr;
+    size_t size = 0, used_bytes = 0;
+    bool retired = false;                        // budget changed: serve no new requests
+    std::map<size_t, size_t> free_by_off;        // offset -> length
+    std::multimap<size_t, size_t> free_by_len;   // length -> offset
+    std::unordered_map<void *, size_t> used;     // pointer -> length
+  } arena;
   std::vector<StreamRec> streams;
   bool sync_ops = false;
   int cus = 0;
@@ -75,6 +89,64 @@ void release_cached(Runtime::Pool &p, bool device, size_t need, size_t limit) {
   }
 }
 
+void arena_erase_free(Runtime::Arena &a, size_t off, size_t len) {
+  a.free_by_off.erase(off);
+  auto range = a.free_by_len.equal_range(len);
+  for (auto it = range.first; it != range.second; ++it)
+    if (it->second == off) {
+      a.free_by_len.erase(it);
+      break;
+    }
+}
+
+void arena_insert_free(Runtime::Arena &a, size_t off, size_t len) {
+  a.free_by_off[off] = len;
+  a.free_by_len.emplace(len, off);
+}
+
+void *arena_alloc(Runtime::Arena &a, size_t want) {
+  auto it = a.free_by_len.lower_bound(want);  // best fit
+  if (it == a.free_by_len.end()) return nullptr;
+  const size_t len = it->first, off = it->second;
+  arena_erase_free(a, off, len);
+  if (len > want) arena_insert_free(a, off + want, len - want);
+  void *ptr = a.base + off;
+  a.used[ptr] = want;
+  a.used_bytes += want;
+  return ptr;
+}
+
+// Returns false when `ptr` does not belong to the arena.
+bool arena_free(Runtime::Arena &a, void *ptr) {
+  auto it = a.used.find(ptr);
+  if (it == a.used.end()) return false;
+  size_t off = (size_t)((char *)ptr - a.base), len = it->second;
+  a.used_bytes -= len;
+  a.used.erase(it);
+  auto next = a.free_by_off.lower_bound(off);
+  if (next != a.free_by_off.end() && next->first == off + len) {  // merge with the range behind
+    const size_t nlen = next->second;
+    arena_erase_free(a, next->first, nlen);
+    len += nlen;
+  }
+  auto prev = a.free_by_off.lower_bound(off);
+  if (prev != a.free_by_off.begin()) {
+    --prev;
+    if (prev->first + prev->second == off) {  // merge with the range in front
+      const size_t poff = prev->first, plen = prev->second;
+      arena_erase_free(a, poff, plen);
+      off = poff;
+      len += plen;
+    }
+  }
+  arena_insert_free(a, off, len);
+  if (a.retired && a.used.empty()) {
+    (void)hipFree(a.base);
+    a = Runtime::Arena();
+  }
+  return true;
+}
+
 void *pool_alloc(Runtime::Pool &p, size_t bytes, bool device, size_t limit) {
   const size_t want = round_size(bytes);
   void *ptr = nullptr;
@@ -102,7 +174,8 @@ void *pool_alloc(Runtime::Pool &p, size_t bytes, bool device, size_t limit) {
   }
   if (ptr) {
     p.in_use += p.block_size[ptr];
-    if (p.in_use > p.peak_in_use) p.peak_in_use = p.in_use;
+    const size_t total = p.in_use + (device ? rt().arena.used_bytes : 0);
+    if (total > p.peak_in_use) p.peak_in_use = total;
   }
   return ptr;
 }
@@ -117,16 +190,48 @@ void pool_free(Runtime::Pool &p, void *ptr) {
 
 }  // namespace
 
+// Creates the arena for the current budget: everything the budget leaves after the
+// blocks already handed out by the pool.  Called with the lock held.
+void arena_open(Runtime &r) {
+  release_cached(r.dev, true, 0, 0);  // nothing stays cached outside the arena
+  if (r.dev_limit <= r.dev.in_use) return;
+  const size_t size = (r.dev_limit - r.dev.in_use) / 65536 * 65536;
+  if (size == 0) return;
+  void *base = nullptr;
+  if (hipMalloc(&base, size) != hipSuccess || !base) {
+    (void)hipGetLastError();
+    return;  // not enough physical memory for the budget: the pool path enforces it instead
+  }
+  r.arena.base = (char *)base;
+  r.arena.size = size;
+  arena_insert_free(r.arena, 0, size);
+}
+
 void *device_alloc(size_t bytes) {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
   r.init();
+  if (r.dev_limit != 0) {
+    if (!r.arena.base) arena_open(r);
+    if (r.arena.base && !r.arena.retired) {
+      void *ptr = arena_alloc(r.arena, round_size(bytes));
+      if (ptr) {
+        const size_t total = r.dev.in_use + r.arena.used_bytes;
+        if (total > r.dev.peak_in_use) r.dev.peak_in_use = total;
+      }
+      return ptr;
+    }
+  }
   return pool_alloc(r.dev, bytes, true, r.dev_limit);
 }
 void device_free(void *p) {
+  if (!p) return;
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
+  if (r.arena.base && arena_free(r.arena, p)) return;
   pool_free(r.dev, p);
+  // a pool block returned while a budget is active must not linger in the cache
+  if (r.dev_limit != 0 && r.arena.base) release_cached(r.dev, true, 0, 0);
 }
 void *pinned_alloc(size_t bytes) {
   Runtime &r = rt();
@@ -311,6 +416,16 @@ extern "C" int DLGpuSetDeviceMemoryLimit(int64_t bytes) {
   std::lock_guard<std::mutex> g(r.mu);
   r.init();
   r.dev_limit = bytes > 0 ? (size_t)bytes : 0;
+  // the arena was sized for the previous budget: retire it (it is handed back
+  // when its last block is freed) and let the next allocation open a new one
+  if (r.arena.base) {
+    if (r.arena.used.empty()) {
+      (void)hipFree(r.arena.base);
+      r.arena = Runtime::Arena();
+    } else {
+      r.arena.retired = true;
+    }
+  }
   if (r.dev_limit) release_cached(r.dev, true, 0, r.dev_limit);
   return 0;
 }
@@ -321,10 +436,10 @@ extern "C" int DLGpuGetDeviceMemoryStats(int64_t *reserved, int64_t *in_use, int
                                          int reset_peak) {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
-  if (reserved) *reserved = (int64_t)r.dev.reserved;
-  if (in_use) *in_use = (int64_t)r.dev.in_use;
+  if (reserved) *reserved = (int64_t)(r.dev.reserved + r.arena.size);
+  if (in_use) *in_use = (int64_t)(r.dev.in_use + r.arena.used_bytes);
   if (peak_in_use) *peak_in_use = (int64_t)r.dev.peak_in_use;
-  if (reset_peak) r.dev.peak_in_use = r.dev.in_use;
+  if (reset_peak) r.dev.peak_in_use = r.dev.in_use + r.arena.used_bytes;
   return 0;
 }
 
