@@ -164,3 +164,51 @@ def test_budget_arena_never_overlaps_and_coalesces():
         whole.free_gpu()
     finally:
         gpu_op.set_device_memory_limit(0)
+
+
+def test_planner_lists_drive_the_step_bit_identically():
+    """A schedule handed over in the planner's wire format (swap list, release
+    list, recomputation list) gives the same bits as the plain executor: the
+    built-in schedule is exported, every ReLU output is additionally released
+    right after its forward use and listed for recomputation before its first
+    backward use."""
+    from tinyflow_amd.SwapExecute import SwapExecutor, schedule_to_wire
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    model, X, y = _shallow_resnet()
+    plain = TrainExecutor(model.loss, 0.01)
+    plain.init_Variable(dict(model.variables))
+    want = [[o.asnumpy() for o in plain.run({model.X: X, model.y_: y})] for _ in range(2)]
+
+    model, X, y = _shallow_resnet()
+    ex = SwapExecutor(model.loss, 0.01, swap=True, min_swap_bytes=1 << 19, prefetch_distance=4)
+    ex.init_Variable(dict(model.variables))
+    ex.run({model.X: X, model.y_: y})            # builds the built-in schedule (and is step 1)
+    pos = {n: i for i, n in enumerate(ex.topo_order)}
+    as_ids = lambda table: {t: [pos[n] for n in ns] for t, ns in table.items()}
+    swap_out, swap_in, release = as_ids(ex.swap_out_at), as_ids(ex.swap_in_at), as_ids(ex.release_at)
+    moved = {i for ids in swap_out.values() for i in ids}
+    recompute = []
+    first_backward = min(pos[n] for n in ex.topo_order if n not in ex.forward_nodes and n.isw not in (1, 2))
+    for n in ex.topo_order:
+        uses = ex.uses[n]
+        if type(n.op).__name__ == "ActivationForwardOp" and n in ex.forward_nodes and pos[n] not in moved:
+            fwd = [u for u in uses if u < first_backward]
+            bwd = [u for u in uses if u >= first_backward]
+            if fwd and bwd and n not in ex.keep:
+                release.setdefault(fwd[-1], []).append(pos[n])
+                recompute.append((bwd[0], pos[n], False))
+    swaps, releases = schedule_to_wire(swap_out, swap_in, release)
+    # a fresh executor fed only with the lists
+    model, X, y = _shallow_resnet()
+    ex2 = SwapExecutor(model.loss, 0.01, swap=True)
+    ex2.init_Variable(dict(model.variables))
+    ex2.set_schedule(swaps, releases, recompute)
+    got = [[o.asnumpy() for o in ex2.run({model.X: X, model.y_: y})] for _ in range(2)]
+    rep = ex2.swap_report()
+    assert rep["offload_bytes"] > 0 and rep["passive_swap_in"] == 0
+    assert recompute and rep["recomputed"] >= len(recompute)
+    for a_step, b_step in zip(want, got):
+        for a, b in zip(a_step, b_step):
+            assert a.tobytes() == b.tobytes()
+    ex.close()
+    ex2.close()

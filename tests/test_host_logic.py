@@ -328,3 +328,19 @@ def test_swap_schedule_orders_every_transfer_around_its_uses():
         if n in keep or n.issgd:
             continue
         assert rel_at[n] == max(uses.get(n, [pos[n]]))
+
+
+def test_planner_wire_format_round_trip():
+    """schedule_to_wire / schedule_from_wire: the planner's list format
+    (reference Scheduler.py:304-331) carries the same schedule as the dicts."""
+    from tinyflow_amd.SwapExecute import schedule_from_wire, schedule_to_wire
+    swap_out = {3: [1, 2], 7: [5]}
+    swap_in = {7: [1], 20: [2, 5]}
+    release = {4: [0], 25: [1, 2, 5]}
+    swaps, releases = schedule_to_wire(swap_out, swap_in, release)
+    assert all(len(m) == 5 and m[1] == 0 and m[4] == 1 for m in swaps)
+    assert [m[2] for m in swaps] == sorted(m[2] for m in swaps)          # issue order = trigger order
+    assert swaps[0] == [1, 0, 3, 0, 1] and [5, 0, 20, 1, 1] in swaps
+    assert releases == [(4, 0), (25, 1), (25, 2), (25, 5)]
+    out2, in2, rel2, rec2 = schedule_from_wire(swaps, releases, [(9, 4, True)])
+    assert out2 == swap_out and in2 == swap_in and rel2 == release and rec2 == {9: [4]}

@@ -208,6 +208,38 @@ def _fit_budget(candidates, pos, last_use, nbytes_of, persistent, budget, steps,
     return sorted(chosen, key=lambda c: order[c[0]])
 
 
+def schedule_to_wire(swap_out, swap_in, release):
+    """The three dicts of ``plan_schedule`` in the planner's wire format
+    (pycode/tinyflow/Scheduler.py:304-331): a swap list of
+    ``[tensor_id, wait_ms, trigger_node_id, to_gpu, 1]`` in issue order and a release
+    list of ``(trigger_node_id, tensor_id)``; ids are positions in the topological order.
+    Takes positions, i.e. dicts ``trigger index -> [tensor index]``."""
+    swaps = []
+    for trigger in sorted(set(swap_out) | set(swap_in)):
+        swaps += [[t, 0, trigger, 0, 1] for t in swap_out.get(trigger, ())]
+        swaps += [[t, 0, trigger, 1, 1] for t in swap_in.get(trigger, ())]
+    releases = [(trigger, t) for trigger in sorted(release) for t in release[trigger]]
+    return swaps, releases
+
+
+def schedule_from_wire(swap_list, release_list, recompute_list=()):
+    """Inverse of ``schedule_to_wire``, also accepting the recomputation list
+    ``(trigger_node_id, tensor_id[, release_flag])``: returns
+    (swap_out, swap_in, release, recompute) as dicts ``trigger index -> [tensor index]``,
+    each list in the order the planner gave.  ``wait_ms`` (the pacing delay the
+    reference's memory thread sleeps, pycode/tinyflow/autodiff.py:90-139) is not
+    used: copies here are ordered by stream events, not by time."""
+    swap_out, swap_in, release, recompute = {}, {}, {}, {}
+    for msg in swap_list:
+        tensor_id, trigger, to_gpu = int(msg[0]), int(msg[2]), int(msg[3])
+        (swap_in if to_gpu else swap_out).setdefault(trigger, []).append(tensor_id)
+    for msg in release_list:
+        release.setdefault(int(msg[0]), []).append(int(msg[1]))
+    for msg in recompute_list:
+        recompute.setdefault(int(msg[0]), []).append(int(msg[1]))
+    return swap_out, swap_in, release, recompute
+
+
 class SwapExecutor(object):
     """SGD step executor that keeps the device footprint small by releasing dead
     values and swapping forward activations to pinned host memory."""
@@ -237,6 +269,20 @@ class SwapExecutor(object):
         self.offloader.start()
         self.prefetcher.start()
         self.stats = {}
+        self.wire_schedule = None
+
+    def set_schedule(self, swap_list, release_list, recompute_list=()):
+        """Run the steps from a planner's lists (the wire format described at
+        ``schedule_from_wire``) instead of the built-in static schedule.  Swaps and
+        releases take effect after their trigger node has been issued, recomputations
+        before it (pycode/tinyflow/autodiff.py:2675-2708, 2814-2835)."""
+        n = len(self.topo_order)
+        sched = schedule_from_wire(swap_list, release_list, recompute_list)
+        for table in sched:
+            for trigger, ids in table.items():
+                assert 0 <= trigger < n and all(0 <= i < n for i in ids), "node id outside the graph"
+        self.wire_schedule = sched
+        self.tensors = None   # re-plan on the next run
 
     def init_Variable(self, feed_dict):
         self.Variable_node_np_value = feed_dict
@@ -256,9 +302,15 @@ class SwapExecutor(object):
         keep = set(n for n in self.topo_order if n.isw in (1, 2)) | {self.targetloss} | self.keep_values
         self.keep = keep
         big = lambda n: self.swap and self.tensors[n].nbytes >= self.min_swap_bytes
-        self.swap_out_at, self.swap_in_at, self.release_at = plan_schedule(
-            self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
-            nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget)
+        self.recompute_at = {}
+        if self.wire_schedule is not None:
+            by_node = [{t: [self.topo_order[i] for i in ids if self.topo_order[i] not in keep]
+                        for t, ids in table.items()} for table in self.wire_schedule]
+            self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = by_node
+        else:
+            self.swap_out_at, self.swap_in_at, self.release_at = plan_schedule(
+                self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
+                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget)
         pos = {n: i for i, n in enumerate(self.topo_order)}
         self.uses = {n: [] for n in self.topo_order}
         for n in self.topo_order:
@@ -314,6 +366,8 @@ class SwapExecutor(object):
         if tensor.state in (MOVING_OUT, MOVING_IN):
             tensor.ready.wait()
             self._check_workers()
+        if tensor.state == FREED and tensor.node.inputs and tensor.node.isw not in (1, 2):
+            self._recompute(tensor.node, self._handles)   # released and not brought back: recompute
         if tensor.state == HOST:   # not prefetched in time: passive swap-in on the compute stream
             self.stats["passive_swap_in"] = self.stats.get("passive_swap_in", 0) + 1
             arr = self._alloc(tensor.shape, tensor.node.name, protect)
@@ -343,13 +397,18 @@ class SwapExecutor(object):
                 t.state = GPU
             else:
                 t.gpu._sync_copyfrom(value)
-        handles = (self.cudnnHandle, self.cublasHandle, self.cudaStream)
+        handles = self._handles = (self.cudnnHandle, self.cublasHandle, self.cudaStream)
+        for t in self.tensors.values():
+            if t.state == HOST and t.node not in self.keep:
+                t.state = FREED   # last step's host copy is stale
         for idx, node in enumerate(self.topo_order):
             t = self.tensors[node]
             if node.isw in (1, 2):
                 pass
             else:
                 self.cursor = idx
+                for again in self.recompute_at.get(idx, ()):
+                    self._recompute(again, handles)
                 input_vals = [self._on_gpu(self.tensors[i], node.inputs) for i in node.inputs]
                 out = None
                 if not node.issgd:
@@ -367,7 +426,8 @@ class SwapExecutor(object):
                 if out is not None:
                     t.gpu, t.state = out, GPU
             for n in self.swap_out_at.get(idx, ()):
-                self.offloader.submit(self.tensors[n], False)
+                if self.tensors[n].state == GPU:
+                    self.offloader.submit(self.tensors[n], False)
             for n in self.swap_in_at.get(idx, ()):
                 tn = self.tensors[n]
                 if tn.state == MOVING_OUT:
@@ -383,9 +443,25 @@ class SwapExecutor(object):
             return [r.asnumpy() for r in result]
         return result
 
+    def _recompute(self, node, handles):
+        """Evaluate ``node`` again from its inputs (a planner released its value and
+        asked for it back by recomputation rather than by a swap-in)."""
+        t = self.tensors[node]
+        if t.state == GPU:
+            return
+        input_vals = [self._on_gpu(self.tensors[i], node.inputs) for i in node.inputs]
+        out = self._alloc(t.shape, node.name + " (recompute)", node.inputs)
+        wanted = node.op.compute(node, input_vals, out, *handles)
+        if wanted:
+            raise MemoryError("%s: %d bytes of device scratch could not be allocated" % (node.name, wanted))
+        t.gpu, t.state = out, GPU
+        self.stats["recomputed"] = self.stats.get("recomputed", 0) + 1
+
     def _release(self, tensor):
         if tensor.state in (MOVING_OUT, MOVING_IN):
             tensor.ready.wait()
+        if tensor.state == HOST:
+            return   # the device copy is gone already; the host copy stays valid for this step
         if tensor.gpu is not None:
             # stream-ordered: kernels already enqueued keep reading the block safely,
             # and whoever receives it next is enqueued behind them
@@ -404,4 +480,4 @@ class SwapExecutor(object):
                 "passive_swap_in": self.stats.get("passive_swap_in", 0),
                 "passive_swap_out": self.stats.get("passive_swap_out", 0),
                 "passive_bytes": self.stats.get("passive_bytes", 0),
-                "prefetch_deferred": self.prefetcher.deferred}
+                "prefetch_deferred": self.prefetcher.deferred, "recomputed": self.stats.get("recomputed", 0)}
