@@ -279,6 +279,35 @@ int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const DLArrayHand
                                     void **Variance_p, void ***list, void **handle,
                                     int *memorytoSaving, void **stream);
 
+/* ----------------------------------------------------- dropout, concatenation */
+
+/* Element-count descriptor that dropout takes in place of the reference's cuDNN
+ * tensor descriptor.  ref: c_runtime_api.h:365-368, gpu_op.cu:3276-3362 */
+int DLGpuGetInputDescriptor(const int *input_shapes, int sizeofshape, int dataformat,
+                            void ***inputd);
+
+/* out = x * keep / (1 - dropout); keep ~ Bernoulli(1 - dropout) drawn from
+ * Philox4x32-10 keyed by `seed` (counter = element index / 4).  The bit mask is
+ * allocated here, published through *reserveSpace_p and listed in *cudnnlist.
+ * ref: c_runtime_api.h:435-443, gpu_op.cu:3547-3640 */
+int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle output, int dataformat,
+                        float dropout, int seed, void **reserveSpace_p, void ***inputd,
+                        void ***cudnnlist, void **handle, int *memorytoSaving, void **stream);
+
+/* dinput = doutput * keep / (1 - dropout); consumes the mask and the list.
+ * ref: c_runtime_api.h:445-449, gpu_op.cu:3647-3693 */
+int DLGpuDropoutBackward(const DLArrayHandle doutput, DLArrayHandle dinput, void **reserveSpace_p,
+                         void ***cudnnlist, void **handle, void **stream);
+
+/* Concatenation of two tensors along axis 1 and the two slices that are its
+ * gradients.  ref: c_runtime_api.h:226-228, gpu_op.cu:967-1084 */
+int DLGpuConcatForward(const DLArrayHandle input1, const DLArrayHandle input2, DLArrayHandle output,
+                       void **stream);
+int DLGpuConcataBackward(const DLArrayHandle input1, const DLArrayHandle input2,
+                         const DLArrayHandle doutput, DLArrayHandle dinput1, void **stream);
+int DLGpuConcatbBackward(const DLArrayHandle input1, const DLArrayHandle input2,
+                         const DLArrayHandle doutput, DLArrayHandle dinput2, void **stream);
+
 /* --------------------------------------------------------------- optimizers */
 
 /* w[i] -= lr * g[i] in place.  ref: c_runtime_api.h:539-543, gpu_op.cu:4600-4625 */

@@ -22,11 +22,16 @@ What pins each function (see tests/test_oracle_*.py):
   pooling                               brute-force loops, sum(dx) == sum(dy), torch CPU
   batch norm                            closed form, sum(dx) = 0, sum(dx*xhat) = 0, torch CPU
   softmax activation backward           Jacobian by finite differences
+  dropout generator (Philox4x32-10)     the known-answer vectors published with Random123;
+                                        keep rate; forward/backward share one mask
+  concatenation                         numpy.concatenate and its slices
 
 Parity unpinned (only real cuDNN 7.6.5 could pin them bit-for-bit): the
 summation order inside the cuDNN/cuBLAS kernels, cudnnPoolingBackward's choice
-among tied maxima, cudnnActivationBackward's value at x == 0.  The tie and zero
-rules used here are stated in max_pool_backward and relu_gradient.
+among tied maxima, cudnnActivationBackward's value at x == 0, and which elements
+cudnnDropoutForward drops for a given seed (its generator is private to cuDNN).
+The tie and zero rules used here are stated in max_pool_backward and relu_gradient,
+the dropout mask definition in dropout_keep_mask.
 """
 import numpy as np
 
@@ -377,3 +382,66 @@ def batch_norm_backward(x, dy, mode, mean=None, istd=None):
     sum_dy = dy.sum(axis=axes, keepdims=True)
     sum_dy_xhat = (dy * xhat).sum(axis=axes, keepdims=True)
     return istd / m * (m * dy - sum_dy - xhat * sum_dy_xhat)
+
+
+# ------------------------------------------------------- dropout, concatenation
+
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy
+    as 1, 2, 3", SC'11).  ``counter``: uint32 array [..., 4]; ``key``: two uint32.
+    Returns uint32 [..., 4].  Pinned by the known-answer vectors published with the
+    Random123 library (tests/test_oracle_ops.py)."""
+    c = np.array(counter, dtype=np.uint64) & np.uint64(0xFFFFFFFF)
+    c0, c1, c2, c3 = c[..., 0], c[..., 1], c[..., 2], c[..., 3]
+    k0, k1 = np.uint64(int(key[0]) & 0xFFFFFFFF), np.uint64(int(key[1]) & 0xFFFFFFFF)
+    m0, m1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0, p1 = m0 * c0, m1 * c2
+        hi0, lo0 = p0 >> np.uint64(32), p0 & mask
+        hi1, lo1 = p1 >> np.uint64(32), p1 & mask
+        c0, c1, c2, c3 = hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0
+        k0 = (k0 + np.uint64(0x9E3779B9)) & mask
+        k1 = (k1 + np.uint64(0xBB67AE85)) & mask
+    return np.stack([c0, c1, c2, c3], axis=-1).astype(np.uint32)
+
+
+def dropout_keep_mask(count, dropout, seed):
+    """Boolean keep-mask of ``count`` elements: element i uses word i % 4 of the
+    Philox block with counter (i // 4, 0, 0, 0) and key (seed, 0) and is kept when
+    that word is >= dropout * 2**32.  This is this build's definition (cuDNN's
+    generator, reference gpu_op.cu:3606-3625, is not reproducible outside cuDNN):
+    parity with the reference's mask bits is unpinned; what is pinned is the
+    generator (known-answer vectors), the keep rate and the fwd/bwd mask identity."""
+    blocks = (count + 3) // 4
+    idx = np.arange(blocks, dtype=np.uint64)
+    ctr = np.stack([idx & np.uint64(0xFFFFFFFF), idx >> np.uint64(32), np.zeros_like(idx), np.zeros_like(idx)], axis=-1)
+    words = philox4x32_10(ctr, (seed, 0)).reshape(-1)[:count]
+    t = float(dropout) * 4294967296.0
+    threshold = np.uint32(0xFFFFFFFF) if t >= 4294967295.0 else np.uint32(int(t))
+    return words >= threshold
+
+
+def dropout_forward(x, dropout, seed):
+    """out = x * keep / (1 - dropout) (cudnnDropoutForward semantics, reference
+    gpu_op.cu:3547-3640); returns (out, keep)."""
+    keep = dropout_keep_mask(x.size, dropout, seed).reshape(x.shape)
+    scale = x.dtype.type(1.0) / (x.dtype.type(1.0) - x.dtype.type(dropout))
+    return np.where(keep, x * scale, np.zeros_like(x)), keep
+
+
+def dropout_backward(dy, keep, dropout):
+    """dx = dy * keep / (1 - dropout) (reference gpu_op.cu:3647-3693)"""
+    scale = dy.dtype.type(1.0) / (dy.dtype.type(1.0) - dy.dtype.type(dropout))
+    return np.where(keep, dy * scale, np.zeros_like(dy))
+
+
+def concat_forward(a, b):
+    """reference gpu_op.cu:967-1003: concatenation along axis 1"""
+    return np.concatenate([a, b], axis=1)
+
+
+def concat_backward(a, b, dout):
+    """reference gpu_op.cu:1006-1084: the two axis-1 slices of dout"""
+    ca = a.shape[1]
+    return np.ascontiguousarray(dout[:, :ca]), np.ascontiguousarray(dout[:, ca:ca + b.shape[1]])

@@ -143,3 +143,88 @@ def test_batch_norm(rt, shape, mode):
     # a second backward without a forward is refused (statistics were consumed)
     with pytest.raises(RuntimeError):
         gpu_op.bn_backward(gx, gdy, gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream)
+
+
+# ------------------------------------------------------- dropout, concatenation
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,p,seed", [((64, 1000), 0.5, 3), ((8, 3, 17, 19), 0.25, 0), ((5,), 0.9, 100),
+                                          ((32, 64, 28, 28), 0.1, 42), ((7, 1, 13), 0.0, 9)])
+def test_dropout_matches_oracle_bit_for_bit(rt, shape, p, seed):
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(1)
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    dy = rng.normal(0, 1, shape).astype(np.float32)
+    want, keep = O.dropout_forward(x, p, seed)
+    inputd = gpu_op.get_input_descriptor(shape, "NCHW")
+    dev_x, dev_dy = ndarray.array(x, rt.ctx), ndarray.array(dy, rt.ctx)
+    out, dx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    reserve, cudnnlist, wanted = gpu_op.dropout_forward(dev_x, out, "NCHW", p, seed, inputd, rt.cudnn, rt.stream)
+    assert wanted == 0
+    assert out.asnumpy().tobytes() == want.tobytes()
+    gpu_op.dropout_backward(dev_dy, dx, reserve, cudnnlist, rt.cudnn, rt.stream)
+    assert dx.asnumpy().tobytes() == O.dropout_backward(dy, keep, p).tobytes()
+
+
+@pytest.mark.gpu
+def test_dropout_backward_needs_its_forward(rt):
+    from tinyflow_amd import gpu_op, ndarray
+    x = ndarray.array(np.ones((4, 8), np.float32), rt.ctx)
+    out = ndarray.empty((4, 8), rt.ctx)
+    inputd = gpu_op.get_input_descriptor((4, 8), "NCHW")
+    reserve, cudnnlist, _ = gpu_op.dropout_forward(x, out, "NCHW", 0.5, 1, inputd, rt.cudnn, rt.stream)
+    gpu_op.dropout_backward(x, out, reserve, cudnnlist, rt.cudnn, rt.stream)
+    with pytest.raises(RuntimeError):   # the list was consumed
+        gpu_op.dropout_backward(x, out, reserve, cudnnlist, rt.cudnn, rt.stream)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sa,sb", [((3, 2, 4, 5), (3, 7, 4, 5)), ((64, 256, 28, 28), (64, 64, 28, 28)),
+                                   ((4, 10), (4, 1)), ((1, 1, 1), (1, 3, 1))])
+def test_concat_forward_and_backward(rt, sa, sb):
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(2)
+    a, b = rng.normal(0, 1, sa).astype(np.float32), rng.normal(0, 1, sb).astype(np.float32)
+    want = O.concat_forward(a, b)
+    da_, db_ = ndarray.array(a, rt.ctx), ndarray.array(b, rt.ctx)
+    out = ndarray.empty(want.shape, rt.ctx)
+    gpu_op.concat_forward(da_, db_, out, rt.stream)
+    assert out.asnumpy().tobytes() == want.tobytes()
+    dout = rng.normal(0, 1, want.shape).astype(np.float32)
+    wa, wb = O.concat_backward(a, b, dout)
+    dev_dout = ndarray.array(dout, rt.ctx)
+    ga, gb = ndarray.empty(sa, rt.ctx), ndarray.empty(sb, rt.ctx)
+    gpu_op.concat_a_backward(da_, db_, dev_dout, ga, rt.stream)
+    gpu_op.concat_b_backward(da_, db_, dev_dout, gb, rt.stream)
+    assert ga.asnumpy().tobytes() == wa.tobytes() and gb.asnumpy().tobytes() == wb.tobytes()
+
+
+@pytest.mark.gpu
+def test_dropout_and_concat_in_a_graph(rt):
+    """y = concat(dropout(x W1), x W2); loss = sum(y * t): gradients through the
+    graph equal the oracle's, with the seed the op drew."""
+    import random
+    from tinyflow_amd import autodiff as ad
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    rng = np.random.RandomState(6)
+    X = rng.normal(0, 1, (16, 12)).astype(np.float32)
+    T = rng.normal(0, 1, (16, 9)).astype(np.float32)
+    W1v, W2v = rng.normal(0, 1, (12, 5)).astype(np.float32), rng.normal(0, 1, (12, 4)).astype(np.float32)
+    x, t = ad.Placeholder("x"), ad.Placeholder("t")
+    W1, W2 = ad.Variable("W1"), ad.Variable("W2")
+    h1 = ad.fullydropout_forward_op(ad.matmul_op(x, W1), "NCHW", 0.4)
+    y = ad.concat_forward_op(h1, ad.matmul_op(x, W2))
+    # scalar loss through the ops that exist on the path: sum over rows then columns
+    loss = ad.reducesumaxiszero_op(ad.reducesumaxiszero_op(ad.mul_op(y, t)))
+    ex = TrainExecutor(loss, 0.0)
+    ex.init_Variable({W1: W1v, W2: W2v})
+    random.seed(123)
+    ex.run({x: X, t: T})
+    seed = h1.seed[0]
+    grads = {v: ex.value_of(g).asnumpy() for v, g in zip(ex.Variable_node_list, ex.Variable_node_grad_list)}
+    a1 = X @ W1v
+    _, keep = O.dropout_forward(a1, 0.4, seed)
+    dy1, dy2 = O.concat_backward(a1, X @ W2v, T)
+    da1 = O.dropout_backward(dy1, keep, 0.4)
+    np.testing.assert_allclose(grads[W1], X.T @ da1, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(grads[W2], X.T @ dy2, rtol=1e-4, atol=1e-5)

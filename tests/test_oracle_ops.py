@@ -369,3 +369,59 @@ def test_adam_and_cross_formulas():
     x, y = rng.uniform(0.1, 1, (4, 3)), np.eye(3)[[0, 2, 1, 1]]
     np.testing.assert_allclose(O.cross(x, y, 0.5), -0.5 * y * np.log(x))
     np.testing.assert_allclose(O.cross_backward(x, y, np.ones_like(x), 0.5), -0.5 * y / x)
+
+
+# ------------------------------------------------------- dropout, concatenation
+
+PHILOX_KAT = [
+    # counter, key, output: known-answer vectors of philox4x32-10 published with the Random123 library
+    ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+    ((0xffffffff,) * 4, (0xffffffff, 0xffffffff), (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+    ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+     (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
+]
+
+
+def test_philox_known_answers():
+    for ctr, key, want in PHILOX_KAT:
+        got = O.philox4x32_10(np.array(ctr, dtype=np.uint32), key)
+        assert tuple(int(v) for v in got) == want
+    # vectorised over a leading axis
+    ctrs = np.array([k[0] for k in PHILOX_KAT[:1]] * 3, dtype=np.uint32)
+    assert O.philox4x32_10(ctrs, (0, 0)).shape == (3, 4)
+
+
+@pytest.mark.parametrize("p", [0.0, 0.1, 0.5, 0.9])
+def test_dropout_mask_rate_scale_and_backward(p):
+    rng = np.random.RandomState(3)
+    x = rng.normal(0, 1, (64, 1000)).astype(np.float32)
+    out, keep = O.dropout_forward(x, p, seed=11)
+    n = x.size
+    assert abs(keep.mean() - (1 - p)) < 4 * np.sqrt(p * (1 - p) / n) + 1e-12
+    assert np.array_equal(out != 0, keep & (x != 0))
+    np.testing.assert_array_equal(out[keep], x[keep] * (np.float32(1) / (np.float32(1) - np.float32(p))))
+    dy = rng.normal(0, 1, x.shape).astype(np.float32)
+    dx = O.dropout_backward(dy, keep, p)
+    # same mask, same scale: <dropout(x), dy> == <x, dropout_backward(dy)>
+    assert abs(np.vdot(out.astype(np.float64), dy) - np.vdot(x.astype(np.float64), dx)) < 1e-6 * n
+    # a different seed gives a different mask, the same seed the same mask
+    assert np.array_equal(keep, O.dropout_forward(x, p, seed=11)[1])
+    if 0 < p < 1:
+        assert not np.array_equal(keep, O.dropout_forward(x, p, seed=12)[1])
+
+
+def test_concat_and_its_gradients():
+    rng = np.random.RandomState(4)
+    a = rng.normal(0, 1, (3, 2, 4, 5)).astype(np.float32)
+    b = rng.normal(0, 1, (3, 7, 4, 5)).astype(np.float32)
+    out = O.concat_forward(a, b)
+    assert out.shape == (3, 9, 4, 5)
+    # the reference kernel's index arithmetic (gpu_op.cu:967-979), element by element
+    count1, count2 = a[0].size, b[0].size
+    flat = out.reshape(-1)
+    for index in range(0, flat.size, 37):
+        i1, i2 = index % (count1 + count2), index // (count1 + count2)
+        want = a.reshape(-1)[i2 * count1 + i1] if i1 < count1 else b.reshape(-1)[i2 * count2 + i1 - count1]
+        assert flat[index] == want
+    da, db = O.concat_backward(a, b, out)
+    assert np.array_equal(da, a) and np.array_equal(db, b)

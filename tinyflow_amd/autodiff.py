@@ -13,6 +13,7 @@ graph, which decides which C entry points run, in which order, on which shapes.
 Every ``compute`` goes through ``gpu_op`` into libc_runtime_api.so; there is no
 numpy branch (the reference keeps one for a subset of ops, autodiff.py:312-779).
 """
+import random
 from functools import reduce
 from operator import add
 
@@ -867,6 +868,136 @@ matmul_op = MatMulOp()
 placeholder_op = PlaceholderOp()
 oneslike_op = OnesLikeOp()
 zeroslike_op = ZerosLikeOp()
+# ------------------------------------------------------- dropout, concatenation
+
+class DropoutForwardOp(Op):
+    """reference autodiff.py:1337-1365.  A fresh seed is drawn from Python's
+    ``random`` module on every evaluation, as there."""
+
+    def __call__(self, node_A, dataformat, dropout):
+        node = Op.__call__(self)
+        node.inputs = [node_A]
+        node.name = "DropoutForward"
+        node.dataformat = dataformat
+        node.dropout = dropout
+        node.seed = [0]
+        node.reserveSpace_p = [0]
+        node.cudnnlist = [0]
+        node.inputd = [0]
+        return node
+
+    def compute(self, node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream, use_numpy=False):
+        _no_numpy(use_numpy)
+        node.seed[0] = random.randint(0, 100)
+        node.reserveSpace_p[0], node.cudnnlist[0], wanted = gpu_op.dropout_forward(
+            input_vals[0], output_val, node.dataformat, node.dropout, node.seed[0], node.inputd[0], cudnnHandle,
+            cudaStream)
+        return wanted
+
+    def gradient(self, node, output_grad):
+        return [dropout_backward_op(output_grad, node.dropout, node.reserveSpace_p, node.cudnnlist)]
+
+    def infer_shape(self, node, input_shapes, cudnnHandle):
+        node.inputd[0] = gpu_op.get_input_descriptor(self._descriptor_shape(input_shapes[0]), node.dataformat)
+        return input_shapes[0]
+
+    @staticmethod
+    def _descriptor_shape(shape):
+        return shape
+
+
+class DropoutBackwardOp(Op):
+    """reference autodiff.py:1368-1387"""
+
+    def __call__(self, node_A, dropout, reserveSpace_p, cudnnlist):
+        node = Op.__call__(self)
+        node.inputs = [node_A]
+        node.name = "DropoutBackward"
+        node.dropout = dropout
+        node.reserveSpace_p = reserveSpace_p
+        node.cudnnlist = cudnnlist
+        return node
+
+    def compute(self, node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream, use_numpy=False):
+        _no_numpy(use_numpy)
+        gpu_op.dropout_backward(input_vals[0], output_val, node.reserveSpace_p[0], node.cudnnlist[0], cudnnHandle,
+                                cudaStream)
+        return 0
+
+    def infer_shape(self, node, input_shapes, cudnnHandle):
+        return input_shapes[0]
+
+
+class FullyDropoutForwardOp(DropoutForwardOp):
+    """Dropout on an (N, F) matrix, described as (N, 1, F) (reference autodiff.py:1390-1422)."""
+
+    def __call__(self, node_A, dataformat, dropout):
+        node = DropoutForwardOp.__call__(self, node_A, dataformat, dropout)
+        node.name = "FullyDropoutForward"
+        return node
+
+    def gradient(self, node, output_grad):
+        return [fullydropout_backward_op(output_grad, node.dropout, node.reserveSpace_p, node.cudnnlist)]
+
+    @staticmethod
+    def _descriptor_shape(shape):
+        return (shape[0], 1, shape[1])
+
+
+class FullyDropoutBackwardOp(DropoutBackwardOp):
+    """reference autodiff.py:1425-1445"""
+
+    def __call__(self, node_A, dropout, reserveSpace_p, cudnnlist):
+        node = DropoutBackwardOp.__call__(self, node_A, dropout, reserveSpace_p, cudnnlist)
+        node.name = "FullyDropoutBackward"
+        return node
+
+
+class ConcatForwardOp(Op):
+    """Concatenation along axis 1 (reference autodiff.py:1935-1956)."""
+
+    def __call__(self, node_A, node_B):
+        node = Op.__call__(self)
+        node.inputs = [node_A, node_B]
+        node.name = "ConcatForward"
+        return node
+
+    def compute(self, node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream, use_numpy=False):
+        _no_numpy(use_numpy)
+        gpu_op.concat_forward(input_vals[0], input_vals[1], output_val, cudaStream)
+        return 0
+
+    def gradient(self, node, output_grad):
+        return [concat_backward_op(node.inputs[0], node.inputs[1], output_grad, 0),
+                concat_backward_op(node.inputs[0], node.inputs[1], output_grad, 1)]
+
+    def infer_shape(self, node, input_shapes, cudnnHandle):
+        shape = list(input_shapes[0])
+        shape[1] = input_shapes[0][1] + input_shapes[1][1]
+        return tuple(shape)
+
+
+class ConcatBackwardOp(Op):
+    """inputs: a, b, d(concat); type 0 / 1 selects the slice for a / b
+    (reference autodiff.py:1959-1984)."""
+
+    def __call__(self, node_A, node_B, node_C, type):
+        node = Op.__call__(self)
+        node.inputs = [node_A, node_B, node_C]
+        node.name = "Concatbackward"
+        node.type = type
+        return node
+
+    def compute(self, node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream, use_numpy=False):
+        _no_numpy(use_numpy)
+        fn = gpu_op.concat_a_backward if node.type == 0 else gpu_op.concat_b_backward
+        fn(input_vals[0], input_vals[1], input_vals[2], output_val, cudaStream)
+        return 0
+
+    def infer_shape(self, node, input_shapes, cudnnHandle):
+        return input_shapes[node.type]
+
+
 reducesumaxiszero_op = ReduceSumAxisZeroOp()
 broadcastto_op = BroadcastToOp()
 broadcastto_gradient_op = BroadcastToGradientOp()
@@ -891,6 +1022,12 @@ bn_forward_op = BNForwardOp()
 bn_backward_op = BNBackwardOp()
 fullybn_forward_op = FullyBNForwardOp()
 sgd_op = SgdOp()
+dropout_forward_op = DropoutForwardOp()
+dropout_backward_op = DropoutBackwardOp()
+fullydropout_forward_op = FullyDropoutForwardOp()
+fullydropout_backward_op = FullyDropoutBackwardOp()
+concat_forward_op = ConcatForwardOp()
+concat_backward_op = ConcatBackwardOp()
 
 
 # ---------------------------------------------------------------- autodiff core

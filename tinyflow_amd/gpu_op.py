@@ -378,6 +378,57 @@ def testPcie():
     check_call(_LIB.testPcie())
 
 
+# ------------------------------------------------------- dropout, concatenation
+
+def get_input_descriptor(input_shapes, dataformat):
+    """reference gpu_op.py:557-570"""
+    fmt = _enum(_DATAFORMAT, dataformat)
+    inputd = _cell(3)
+    check_call(_LIB.DLGpuGetInputDescriptor(c_array(ctypes.c_int, input_shapes), len(input_shapes), fmt, inputd))
+    return inputd
+
+
+def dropout_forward(input, output, dataformat, dropout, seed, inputd, cudnnHandle, cudaStream):
+    """Returns (reserveSpace_p, cudnnlist, bytes wanted); reference gpu_op.py:657-685."""
+    _nd_args(input, output)
+    fmt = _enum(_DATAFORMAT, dataformat)
+    assert seed >= 0
+    reserveSpace_p = _cell(2)
+    cudnnlist = _cell(3)
+    wanted = ctypes.c_int(0)
+    check_call(_LIB.DLGpuDropoutForward(input.handle, output.handle, fmt, ctypes.c_float(dropout),
+                                        ctypes.c_int(seed), reserveSpace_p, inputd, cudnnlist, cudnnHandle,
+                                        ctypes.byref(wanted), cudaStream))
+    return reserveSpace_p, cudnnlist, wanted.value
+
+
+def dropout_backward(doutput, dinput, reserveSpace_p, cudnnlist, cudnnHandle, cudaStream):
+    """reference gpu_op.py:688-692"""
+    _nd_args(doutput, dinput)
+    check_call(_LIB.DLGpuDropoutBackward(doutput.handle, dinput.handle, reserveSpace_p, cudnnlist,
+                                         cudnnHandle, cudaStream))
+
+
+def concat_forward(in_arr_a, in_arr_b, out_arr, cudaStream):
+    """reference gpu_op.py:746-751"""
+    _nd_args(in_arr_a, in_arr_b, out_arr)
+    check_call(_LIB.DLGpuConcatForward(in_arr_a.handle, in_arr_b.handle, out_arr.handle, cudaStream))
+
+
+def concat_a_backward(in_arr_a, in_arr_b, out_arr, din_arr_a, cudaStream):
+    """reference gpu_op.py:752-758; ``out_arr`` is the gradient of the concatenation"""
+    _nd_args(in_arr_a, in_arr_b, out_arr, din_arr_a)
+    check_call(_LIB.DLGpuConcataBackward(in_arr_a.handle, in_arr_b.handle, out_arr.handle, din_arr_a.handle,
+                                         cudaStream))
+
+
+def concat_b_backward(in_arr_a, in_arr_b, out_arr, din_arr_b, cudaStream):
+    """reference gpu_op.py:760-768"""
+    _nd_args(in_arr_a, in_arr_b, out_arr, din_arr_b)
+    check_call(_LIB.DLGpuConcatbBackward(in_arr_a.handle, in_arr_b.handle, out_arr.handle, din_arr_b.handle,
+                                         cudaStream))
+
+
 # --------------------------------------------------- allocator budget (extension)
 
 def set_device_memory_limit(nbytes):
