@@ -20,9 +20,9 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libc_runtime_api.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-# packed-fp32 code generation is switched off for device code (see the build
-# notes of this pool: some packed fp32 forms miscompute); the host pass does not
-# know the feature and says so, which is harmless.
+# Packed-fp32 code generation (v_pk_*_f32) is switched off for device code: some
+# of its forms have produced wrong results on this hardware without any error.
+# The host pass does not know the feature and says so, which is harmless.
 CXXFLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
