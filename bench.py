@@ -211,6 +211,9 @@ def main():
     ap.add_argument("--bn-mode", default="pre_activation", choices=["pre_activation", "spatial"],
                     help="pre_activation is what every model graph of the reference passes")
     ap.add_argument("--config", default="resnet50", choices=["resnet50", "vgg16", "lenet5", "mlp", "resnet152"])
+    ap.add_argument("--no-recompute", action="store_true",
+                    help="with --mem-limit-gb: move every scheduled activation over PCIe instead of recomputing "
+                         "batch-norm / ReLU outputs in the backward pass")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--no-kernel-events", action="store_true",
@@ -244,7 +247,8 @@ def main():
         from tinyflow_amd.SwapExecute import SwapExecutor
         limit = int(args.mem_limit_gb * (1 << 30))
         gpu_op.set_device_memory_limit(limit)
-        ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=int(0.95 * limit), prefetch_distance=12)
+        ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=int(0.95 * limit), prefetch_distance=12,
+                          recompute=not args.no_recompute)
     else:
         ex = TrainExecutor(model.loss, 0.01)
     ex.init_Variable(dict(model.variables))
@@ -351,6 +355,7 @@ def main():
             "pcie_GBps_over_step": (moved["offload_bytes"] + moved["prefetch_bytes"] + moved["passive_bytes"])
                                    / wall / 1e9,
             "passive_swap_in": moved["passive_swap_in"], "passive_swap_out": moved["passive_swap_out"],
+            "recomputed_per_step": moved["recomputed"] / args.steps,
         }
         ex.close()
     if not args.no_cpu_baseline:

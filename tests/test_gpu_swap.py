@@ -47,13 +47,14 @@ def test_pcie_probe_runs():
 def test_swapped_step_is_bit_identical_to_plain_step():
     from tinyflow_amd.SwapExecute import SwapExecutor
     from tinyflow_amd.TrainExecute import TrainExecutor
-    results = []
-    for kind in ("plain", "release", "swap"):
+    results, moved = [], {}
+    for kind in ("plain", "release", "swap", "recompute"):
         model, X, y = _shallow_resnet()
         if kind == "plain":
             ex = TrainExecutor(model.loss, 0.01)
         else:
-            ex = SwapExecutor(model.loss, 0.01, swap=(kind == "swap"), min_swap_bytes=1 << 12, prefetch_distance=4)
+            ex = SwapExecutor(model.loss, 0.01, swap=(kind != "release"), min_swap_bytes=1 << 12, prefetch_distance=4,
+                              recompute=(kind == "recompute"))
             ex.keep_values = set(ex.Variable_node_grad_list)
         ex.init_Variable(dict(model.variables))
         feed = {model.X: X, model.y_: y}
@@ -62,13 +63,16 @@ def test_swapped_step_is_bit_identical_to_plain_step():
             out = ex.run(feed)
             grads = [ex.value_of(g).asnumpy() for g in ex.Variable_node_grad_list]
             steps.append(([o.asnumpy() for o in out], grads))
-        if kind == "swap":
+        if kind in ("swap", "recompute"):
             rep = ex.swap_report()
             assert rep["offload_bytes"] > 0 and rep["prefetch_bytes"] == rep["offload_bytes"]
             assert rep["passive_swap_in"] == 0
+            assert (rep["recomputed"] > 0) == (kind == "recompute")
+            moved[kind] = rep["offload_bytes"]
         if kind != "plain":
             ex.close()
         results.append(steps)
+    assert moved["recompute"] < 0.7 * moved["swap"]   # normalisation / activation outputs no longer travel
     for other in results[1:]:
         for (out_a, g_a), (out_b, g_b) in zip(results[0], other):
             for a, b in zip(out_a + g_a, out_b + g_b):

@@ -302,7 +302,8 @@ def test_swap_schedule_orders_every_transfer_around_its_uses():
     topo = swapsgd(ad.find_topo_sort(getcomputelist(variables, grads, 0.1)))
     forward = set(ad.find_topo_sort([model.loss]))
     keep = set(variables) | {model.X, model.y_, model.loss}
-    swap_out, swap_in, release = plan_schedule(topo, forward, keep, lambda n: True, 2)
+    swap_out, swap_in, release, recompute = plan_schedule(topo, forward, keep, lambda n: True, 2)
+    assert recompute == {}
     pos = {n: i for i, n in enumerate(topo)}
     uses = {}
     for n in topo:

@@ -130,42 +130,79 @@ class MemoryManager(threading.Thread):
         self.bytes_moved += tensor.nbytes
 
 
-def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of=None, budget=None):
-    """vDNN-style static schedule.
+def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of=None, budget=None,
+                  recomputable=None):
+    """Static schedule in the manner of vDNN, optionally with recomputation.
 
-    Returns (swap_out, swap_in, release), each a dict ``trigger index -> [node]``:
-    after the node at ``trigger`` has been issued, the listed tensors are swapped
-    out / prefetched / released.  A forward value that backward uses again is
-    swapped out after its last forward use and prefetched ``prefetch_distance``
-    nodes before its first backward use; every value is released after its last
-    use.  ``keep`` (variables, feeds, the loss) is never moved or released.
+    Returns (swap_out, swap_in, release, recompute), each a dict ``trigger index ->
+    [node]``: after the node at ``trigger`` has been issued, the listed tensors are
+    swapped out / prefetched / released; the tensors of ``recompute`` are evaluated
+    again *before* the trigger node.  ``keep`` (variables, feeds, the loss) is never
+    moved or released.
 
-    With ``budget`` (bytes) and ``nbytes_of`` the schedule only moves as many
-    tensors as it takes for the simulated footprint to fit: it walks the live-bytes
-    timeline and, while its peak is above the budget, offloads the candidate that
-    spans the peak with the largest bytes x absence product (early, large
-    activations first, as vDNN does).  Without a budget every candidate moves.
+    * Every value is released after its last use.
+    * ``recomputable(node)`` marks forward values that are cheap to evaluate again
+      (normalisation, activation).  Such a value is released after its last forward
+      use and recomputed before its first backward use, provided that this does not
+      chain more than two recomputations (its inputs are swapped or kept values, or
+      values recomputed directly from those).  A recomputation is an additional,
+      earlier use of its inputs, which the prefetch points below take into account.
+    * A forward value that backward uses again and is not recomputed is swapped out
+      after its last forward use and prefetched ``prefetch_distance`` nodes before
+      its first backward use.  With ``budget`` (bytes) and ``nbytes_of`` only as
+      many tensors move as it takes for the simulated footprint to fit: while the
+      peak of the live-bytes timeline is above the budget, the candidate spanning
+      the peak with the largest bytes x absence product goes (early, large
+      activations first).  Without a budget every candidate moves.
     """
     pos = {n: i for i, n in enumerate(topo_order)}
-    uses = {}
+    uses = {n: [] for n in topo_order}
     for n in topo_order:
         for inp in n.inputs:
-            uses.setdefault(inp, []).append(pos[n])
+            uses[inp].append(pos[n])
     first_backward = min((pos[n] for n in topo_order if n not in forward_nodes and n.isw not in (1, 2)),
                          default=len(topo_order))
-    release, last_use, candidates = {}, {}, []
-    for n in topo_order:
-        if n in keep or n.issgd:
+    movable = [n for n in topo_order if n not in keep and not n.issgd]
+
+    # which forward values are recomputed (decided in forward order: depth of the chain)
+    depth = {}
+    if recomputable is not None:
+        for n in movable:
+            if n not in forward_nodes or not recomputable(n) or not n.inputs:
+                continue
+            if not any(u >= first_backward for u in uses[n]) or not any(u < first_backward for u in uses[n]):
+                continue
+            d = 1 + max((depth.get(i, 0) for i in n.inputs), default=0)
+            if d <= 2:
+                depth[n] = d
+    # recompute triggers, consumers first, so that the extra use of an input is known
+    # when the input's own trigger is chosen
+    extra = {n: [] for n in topo_order}
+    recompute, recompute_at = {}, {}
+    for n in reversed(movable):
+        if n not in depth:
             continue
-        use_idx = sorted(uses.get(n, []))
-        last = use_idx[-1] if use_idx else pos[n]
+        later = [u for u in uses[n] + extra[n] if u >= first_backward]
+        trigger = min(later)
+        recompute_at[n] = trigger
+        recompute.setdefault(trigger, []).append(n)
+        for inp in n.inputs:
+            extra[inp].append(trigger)
+    for trigger in recompute:   # producers before consumers
+        recompute[trigger].sort(key=lambda n: pos[n])
+
+    release, last_use, candidates = {}, {}, []
+    for n in movable:
+        all_uses = sorted(uses[n] + extra[n])
+        last = all_uses[-1] if all_uses else pos[n]
         last_use[n] = last
         release.setdefault(last, []).append(n)
-        if n not in forward_nodes or not min_bytes_of(n):
+        fwd_uses = [u for u in all_uses if u < first_backward]
+        bwd_uses = [u for u in all_uses if u >= first_backward]
+        if n in depth:
+            release.setdefault(fwd_uses[-1], []).append(n)
             continue
-        fwd_uses = [u for u in use_idx if u < first_backward]
-        bwd_uses = [u for u in use_idx if u >= first_backward]
-        if not bwd_uses:
+        if n not in forward_nodes or not min_bytes_of(n) or not bwd_uses:
             continue
         out_at = fwd_uses[-1] if fwd_uses else pos[n]
         in_at = max(bwd_uses[0] - prefetch_distance, first_backward - 1, out_at + 1)
@@ -173,25 +210,29 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
             continue  # needed again too soon for a round trip to pay
         candidates.append((n, out_at, in_at))
     if budget is not None:
-        candidates = _fit_budget(candidates, pos, last_use, nbytes_of, sum(nbytes_of(n) for n in keep),
+        absent = {n: (max(u for u in uses[n] if u < first_backward), recompute_at[n]) for n in depth}
+        candidates = _fit_budget(candidates, pos, last_use, absent, nbytes_of, sum(nbytes_of(n) for n in keep),
                                  budget, len(topo_order), prefetch_distance)
     swap_out, swap_in = {}, {}
     for n, out_at, in_at in candidates:
         swap_out.setdefault(out_at, []).append(n)
         swap_in.setdefault(in_at, []).append(n)
-    return swap_out, swap_in, release
+    return swap_out, swap_in, release, recompute
 
 
-def _fit_budget(candidates, pos, last_use, nbytes_of, persistent, budget, steps, lag):
+def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget, steps, lag):
     """Smallest greedy subset of ``candidates`` whose removal brings the simulated
     footprint under ``budget``.  A swapped-out block is counted as resident until
-    ``lag`` nodes after its trigger (its copy has to finish first)."""
+    ``lag`` nodes after its trigger (its copy has to finish first); ``absent`` maps a
+    recomputed value to the (release, recompute) indices between which it is gone."""
     live = np.zeros(steps + 1, dtype=np.int64)
     for n, born in pos.items():
         if n in last_use:
             live[born] += nbytes_of(n)
             live[last_use[n] + 1] -= nbytes_of(n)
     live = np.cumsum(live)[:steps] + persistent
+    for n, (gone, back) in absent.items():
+        live[gone + 1:back] -= nbytes_of(n)
     chosen, remaining = [], list(candidates)
     while remaining:
         peak = int(np.argmax(live))
@@ -245,7 +286,7 @@ class SwapExecutor(object):
     values and swapping forward activations to pinned host memory."""
 
     def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), swap=True, min_swap_bytes=1 << 20,
-                 prefetch_distance=8, memory_budget=None):
+                 prefetch_distance=8, memory_budget=None, recompute=False):
         self.targetloss = targetloss
         self.ctx = ctx
         self.Variable_node_list = ad.get_Variable_node_list(targetloss)
@@ -258,6 +299,7 @@ class SwapExecutor(object):
         self.min_swap_bytes = min_swap_bytes
         self.prefetch_distance = prefetch_distance
         self.memory_budget = memory_budget   # bytes the schedule plans for; None: move every candidate
+        self.recompute = recompute           # evaluate normalisation / activation outputs again instead of moving them
         self.cudaStream = gpu_op.create_cudaStream()
         self.cudnnHandle = gpu_op.create_cudnnHandle(self.cudaStream)
         self.cublasHandle = gpu_op.create_cublasHandle(self.cudaStream)
@@ -308,9 +350,11 @@ class SwapExecutor(object):
                         for t, ids in table.items()} for table in self.wire_schedule]
             self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = by_node
         else:
-            self.swap_out_at, self.swap_in_at, self.release_at = plan_schedule(
+            cheap = (ad.BNForwardOp, ad.ActivationForwardOp, ad.ReluOp)
+            again = (lambda n: isinstance(n.op, cheap)) if (self.swap and self.recompute) else None
+            self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = plan_schedule(
                 self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
-                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget)
+                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again)
         pos = {n: i for i, n in enumerate(self.topo_order)}
         self.uses = {n: [] for n in self.topo_order}
         for n in self.topo_order:
