@@ -345,3 +345,57 @@ def test_planner_wire_format_round_trip():
     assert releases == [(4, 0), (25, 1), (25, 2), (25, 5)]
     out2, in2, rel2, rec2 = schedule_from_wire(swaps, releases, [(9, 4, True)])
     assert out2 == swap_out and in2 == swap_in and rel2 == release and rec2 == {9: [4]}
+
+
+def test_recompute_schedule_invariants():
+    """plan_schedule with recomputation on a shallow bottleneck ResNet: batch-norm and
+    activation outputs are rebuilt instead of moved, every recomputation comes no
+    later than the first backward use, its inputs are back on the device by then,
+    chains are at most two long, and producers are rebuilt before their consumers."""
+    from tinyflow_amd import autodiff as ad, models
+    from tinyflow_amd.SwapExecute import plan_schedule
+    from tinyflow_amd.TrainExecute import getcomputelist, swapsgd
+    rng = np.random.RandomState(0)
+    model = models.resnet(rng, [1, 1, 1, 1], 4, image=32, n_class=10, width=8)
+    variables = ad.get_Variable_node_list(model.loss)
+    variables.reverse()
+    grads = ad.gradients(model.loss, variables)
+    topo = swapsgd(ad.find_topo_sort(getcomputelist(variables, grads, 0.1)))
+    forward = set(ad.find_topo_sort([model.loss]))
+    keep = set(n for n in topo if n.isw in (1, 2)) | {model.loss}
+    cheap = lambda n: isinstance(n.op, (ad.BNForwardOp, ad.ActivationForwardOp))
+    swap_out, swap_in, release, recompute = plan_schedule(topo, forward, keep, lambda n: True, 4, recomputable=cheap)
+    pos = {n: i for i, n in enumerate(topo)}
+    uses = {n: [] for n in topo}
+    for n in topo:
+        for inp in n.inputs:
+            uses[inp].append(pos[n])
+    first_backward = min(pos[n] for n in topo if n not in forward and n.isw not in (1, 2))
+    rec_at = {n: t for t, ns in recompute.items() for n in ns}
+    out_at = {n: t for t, ns in swap_out.items() for n in ns}
+    in_at = {n: t for t, ns in swap_in.items() for n in ns}
+    assert rec_at, "nothing is recomputed"
+    assert not set(rec_at) & set(out_at), "a recomputed value is also swapped"
+    n_bn = sum(isinstance(n.op, ad.BNForwardOp) for n in rec_at)
+    n_act = sum(isinstance(n.op, ad.ActivationForwardOp) for n in rec_at)
+    assert n_bn > 0 and n_act > 0
+
+    def chain(n):
+        return 0 if n not in rec_at else 1 + max(chain(i) for i in n.inputs)
+
+    for n, t in rec_at.items():
+        assert cheap(n) and n in forward and n not in keep
+        bwd = [u for u in uses[n] if u >= first_backward]
+        assert t >= first_backward and t <= min(bwd)
+        assert 1 <= chain(n) <= 2
+        for inp in n.inputs:
+            if inp in rec_at:
+                assert rec_at[inp] <= t
+                if rec_at[inp] == t:   # same trigger: the producer is listed first
+                    order = recompute[t]
+                    assert order.index(inp) < order.index(n)
+            if inp in in_at:
+                assert in_at[inp] < t, "input is prefetched only after the recomputation needs it"
+        # released once after the forward pass and once for good
+        rel = sorted(t2 for t2, ns in release.items() if n in ns)
+        assert len(rel) == 2 and rel[0] < first_backward <= rel[1] and rel[0] < t <= rel[1]
