@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   save_istd[l] = istd;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) __builtin_nontemporal_store((v[n] - mean) * istd, y + (int64_t)n * L + l);
+    if (n < N) y[(int64_t)n * L + l] = (v[n] - mean) * istd;
 }
 
 // any N: three sweeps over the column (the second and third hit the cache)
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
   const float scale = istd / m;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) __builtin_nontemporal_store(scale * (m * g[n] - s1 - xh[n] * s2), dx + (int64_t)n * L + l);
+    if (n < N) dx[(int64_t)n * L + l] = scale * (m * g[n] - s1 - xh[n] * s2);
 }
 
 __global__ __launch_bounds__(kThreads) void bn_pa_backward_stream_kernel(const float *__restrict__ x,

@@ -2,8 +2,8 @@
 //
 // Each workgroup owns one contiguous run of 1024 16-byte vectors (16 KiB per
 // operand): every lane issues four independent vector loads per operand before
-// the first store, and loads and stores carry the non-temporal hint, since each
-// byte is touched once.  Contiguous runs per workgroup keep a workgroup's
+// the first store, and the loads carry the non-temporal hint, since each byte is
+// read once.  Contiguous runs per workgroup keep a workgroup's
 // traffic inside few DRAM pages; measured on MI355X this moves 12-byte-per-
 // element work at 5.6-6.5 TB/s, against 4.6-4.9 TB/s for a grid-stride loop.
 #pragma once
@@ -20,7 +20,10 @@ constexpr int kVecPerBlock = kThreads * kUnroll;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline f32x4 load_stream(const f32x4 *p) { return __builtin_nontemporal_load(p); }
-__device__ inline void store_stream(f32x4 v, f32x4 *p) { __builtin_nontemporal_store(v, p); }
+// results are stored with the default policy: the next kernel usually reads them
+// back, and a plain store leaves them in the last-level cache (measured +0.5 % on the
+// ResNet-50 step against a non-temporal store)
+__device__ inline void store_stream(f32x4 v, f32x4 *p) { *p = v; }
 
 template <class F>
 __device__ inline f32x4 apply4(const F &f, const f32x4 &a, const f32x4 &b) {
