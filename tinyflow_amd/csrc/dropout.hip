@@ -15,9 +15,11 @@
 // reproduces it; cuDNN's own generator is not reproducible outside cuDNN.
 //
 // Concatenation along axis 1 replaces src/gpu_op.cu:967-1084.
+#include "gemm_core.h"
 #include "internal.h"
 
 using namespace tf;
+using tf::gemm::FastDiv;
 
 namespace {
 
@@ -96,24 +98,25 @@ __global__ __launch_bounds__(kThreads) void dropout_kernel(const float *__restri
 }
 
 // out[o, :] = [a[o, :ca], b[o, :cb]] with ca / cb elements per outer index
-__global__ __launch_bounds__(kThreads) void concat_kernel(const float *__restrict__ a, int64_t ca,
-                                                         const float *__restrict__ b, int64_t cb,
-                                                         float *__restrict__ out, int64_t total) {
-  const int64_t row = ca + cb;
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-    const int64_t o = i / row, j = i - o * row;
-    out[i] = j < ca ? a[o * ca + j] : b[o * cb + (j - ca)];
+__global__ __launch_bounds__(kThreads) void concat_kernel(const float *__restrict__ a, uint32_t ca,
+                                                         const float *__restrict__ b, uint32_t cb, FastDiv row,
+                                                         float *__restrict__ out, uint32_t total) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    uint32_t o, j;
+    row.divmod(i, o, j);
+    out[i] = j < ca ? a[(int64_t)o * ca + j] : b[(int64_t)o * cb + (j - ca)];
   }
 }
 
 // din[o, :] = dout[o, offset : offset + width]
 __global__ __launch_bounds__(kThreads) void slice_kernel(const float *__restrict__ dout, int64_t row, int64_t offset,
-                                                        int64_t width, float *__restrict__ din, int64_t total) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-    const int64_t o = i / width, j = i - o * width;
-    din[i] = dout[o * row + offset + j];
+                                                        FastDiv width, float *__restrict__ din, uint32_t total) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    uint32_t o, j;
+    width.divmod(i, o, j);
+    din[i] = dout[(int64_t)o * row + offset + j];
   }
 }
 
@@ -225,9 +228,11 @@ extern "C" int DLGpuConcatForward(const DLArrayHandle input1, const DLArrayHandl
   TF_REQUIRE(on_gpu(output) && numel(output) == numel(input1) + numel(input2), "output has the wrong size");
   hipStream_t s = stream_of(stream);
   const int64_t total = numel(output);
+  TF_REQUIRE(total < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   if (total > 0)
-    hipLaunchKernelGGL(concat_kernel, dim3(grid_for(total)), dim3(kThreads), 0, s, (const float *)input1->data, ca,
-                       (const float *)input2->data, cb, (float *)output->data, total);
+    hipLaunchKernelGGL(concat_kernel, dim3(grid_for(total)), dim3(kThreads), 0, s, (const float *)input1->data,
+                       (uint32_t)ca, (const float *)input2->data, (uint32_t)cb, FastDiv((uint32_t)(ca + cb)),
+                       (float *)output->data, (uint32_t)total);
   return finish(s, "DLGpuConcatForward");
 }
 
@@ -240,9 +245,10 @@ static int concat_backward(const DLArray *input1, const DLArray *input2, const D
   TF_REQUIRE(on_gpu(dinput) && numel(dinput) == outer * width, "dinput has the wrong size");
   hipStream_t s = stream_of(stream);
   const int64_t total = outer * width;
+  TF_REQUIRE(numel(doutput) < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   if (total > 0)
     hipLaunchKernelGGL(slice_kernel, dim3(grid_for(total)), dim3(kThreads), 0, s, (const float *)doutput->data,
-                       ca + cb, second ? ca : 0, width, (float *)dinput->data, total);
+                       ca + cb, second ? ca : 0, FastDiv((uint32_t)width), (float *)dinput->data, (uint32_t)total);
   return finish(s, what);
 }
 

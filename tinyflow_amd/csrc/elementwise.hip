@@ -11,9 +11,11 @@
 // :4538-4597 (cross), :4600-4625 (SGD); one thread per element, 1024-thread
 // blocks capped at 4096 blocks there.
 #include "ew_core.h"
+#include "gemm_core.h"
 #include "internal.h"
 
 using namespace tf;
+using tf::gemm::FastDiv;
 
 using namespace tf::ew;
 
@@ -33,23 +35,28 @@ struct OpSgd { float lr; __device__ float operator()(float a, float b) const { r
 // a = x (probabilities), b = y (labels)
 struct OpCross { float s; __device__ float operator()(float a, float b) const { return logf(a) * b * (-1.f) * s; } };
 
-// out[i] = in[i % in_count]
-__global__ __launch_bounds__(kThreads) void broadcast_tail_kernel(const float *__restrict__ in, int in_count,
-                                                                 float *__restrict__ out, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
-    out[i] = in[(int)(i % in_count)];
+// out[i] = in[i % in_count].  Indices are 32-bit and divided by magic numbers: a
+// 64-bit integer division per element would cost more than the memory traffic.
+__global__ __launch_bounds__(kThreads) void broadcast_tail_kernel(const float *__restrict__ in, FastDiv in_count,
+                                                                 float *__restrict__ out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
+    uint32_t q, r;
+    in_count.divmod(i, q, r);
+    out[i] = in[r];
+  }
 }
 
 // out[n, c, inner] = in[c]; one float4 per lane when inner % 4 == 0
 template <bool VEC>
-__global__ __launch_bounds__(kThreads) void broadcast_channel_kernel(const float *__restrict__ in, int C,
-                                                                    int inner, float *__restrict__ out,
-                                                                    int64_t n_units) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  const int units_per_row = VEC ? inner / 4 : inner;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n_units; i += stride) {
-    const int c = (int)((i / units_per_row) % C);
+__global__ __launch_bounds__(kThreads) void broadcast_channel_kernel(const float *__restrict__ in, FastDiv channels,
+                                                                    FastDiv units_per_row,
+                                                                    float *__restrict__ out, uint32_t n_units) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n_units; i += stride) {
+    uint32_t row, img, c;
+    row = units_per_row.div(i);
+    channels.divmod(row, img, c);
     const float v = in[c];
     if (VEC) reinterpret_cast<float4 *>(out)[i] = make_float4(v, v, v, v);
     else out[i] = v;
@@ -199,8 +206,9 @@ extern "C" int DLGpuBroadcastTo0(const DLArrayHandle in, DLArrayHandle out, void
   }
   hipStream_t s = stream_of(stream);
   if (n == 0) return 0;
+  TF_REQUIRE(n < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   hipLaunchKernelGGL(broadcast_tail_kernel, dim3(grid_for(n)), dim3(kThreads), 0, s, (const float *)in->data,
-                     (int)in_count, (float *)out->data, n);
+                     FastDiv((uint32_t)in_count), (float *)out->data, (uint32_t)n);
   return finish(s, "DLGpuBroadcastTo0");
 }
 
@@ -214,14 +222,17 @@ extern "C" int DLGpuBroadcastTo1(const DLArrayHandle in, DLArrayHandle out, void
   TF_REQUIRE(inner <= INT32_MAX, "inner extent too large");
   hipStream_t s = stream_of(stream);
   if (n == 0) return 0;
-  const int C = (int)out->shape[1];
+  TF_REQUIRE(n < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
+  const FastDiv channels((uint32_t)out->shape[1]);
   if (inner % 4 == 0 && aligned16(out->data)) {
     const int64_t units = n / 4;
     hipLaunchKernelGGL(broadcast_channel_kernel<true>, dim3(grid_for(units)), dim3(kThreads), 0, s,
-                       (const float *)in->data, C, (int)inner, (float *)out->data, units);
+                       (const float *)in->data, channels, FastDiv((uint32_t)(inner / 4)), (float *)out->data,
+                       (uint32_t)units);
   } else {
     hipLaunchKernelGGL(broadcast_channel_kernel<false>, dim3(grid_for(n)), dim3(kThreads), 0, s,
-                       (const float *)in->data, C, (int)inner, (float *)out->data, n);
+                       (const float *)in->data, channels, FastDiv((uint32_t)inner), (float *)out->data,
+                       (uint32_t)n);
   }
   return finish(s, "DLGpuBroadcastTo1");
 }

@@ -10,9 +10,15 @@
 // that cover it and name it.  A gather needs no atomics, so the result is
 // deterministic even when windows overlap (3x3 stride 2), and the forward output
 // y is not needed.
+//
+// Element indices are 32-bit (tensors hold fewer than 2^31 elements) and are split
+// into (plane, row, column) with magic-number divisions: 64-bit integer division,
+// which the compiler emits for int64 indices, costs more than the memory traffic.
+#include "gemm_core.h"
 #include "internal.h"
 
 using namespace tf;
+using tf::gemm::FastDiv;
 
 namespace {
 
@@ -21,19 +27,19 @@ constexpr int kThreads = 256;
 struct PoolParams {
   int C, H, W, P, Q;
   int pad_h, pad_w, u, v, fh, fw;
+  FastDiv div_pq, div_q, div_hw, div_w;
 };
 
 template <bool MAX>
 __global__ __launch_bounds__(kThreads) void pool_forward_kernel(const float *__restrict__ x, float *__restrict__ y,
-                                                               PoolParams pp, int64_t total) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-    const int q = (int)(i % pp.Q);
-    const int64_t t = i / pp.Q;
-    const int p = (int)(t % pp.P);
-    const int64_t nc = t / pp.P;
-    const float *plane = x + nc * pp.H * pp.W;
-    const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+                                                               PoolParams pp, uint32_t total) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    uint32_t nc, pix, p, q;
+    pp.div_pq.divmod(i, nc, pix);
+    pp.div_q.divmod(pix, p, q);
+    const int h0 = (int)p * pp.u - pp.pad_h, w0 = (int)q * pp.v - pp.pad_w;
+    const float *plane = x + (int64_t)nc * pp.H * pp.W;
     float acc = MAX ? -INFINITY : 0.f;
     for (int r = 0; r < pp.fh; ++r) {
       const int h = h0 + r;
@@ -58,15 +64,14 @@ __device__ inline int ceil_div_floor0(int a, int b) {  // ceil(a / b) clamped at
 // holds the window's first maximum in row-major order.
 __global__ __launch_bounds__(kThreads) void pool_argmax_kernel(const float *__restrict__ x,
                                                               unsigned char *__restrict__ tap, PoolParams pp,
-                                                              int64_t total) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-    const int q = (int)(i % pp.Q);
-    const int64_t t = i / pp.Q;
-    const int p = (int)(t % pp.P);
-    const int64_t nc = t / pp.P;
-    const float *plane = x + nc * pp.H * pp.W;
-    const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+                                                              uint32_t total) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    uint32_t nc, pix, p, q;
+    pp.div_pq.divmod(i, nc, pix);
+    pp.div_q.divmod(pix, p, q);
+    const int h0 = (int)p * pp.u - pp.pad_h, w0 = (int)q * pp.v - pp.pad_w;
+    const float *plane = x + (int64_t)nc * pp.H * pp.W;
     float best = -INFINITY;
     int arg = 255;  // stays 255 when the window holds no comparable value (all NaN)
     for (int r = 0; r < pp.fh; ++r) {
@@ -92,13 +97,13 @@ template <bool MAX>
 __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned char *__restrict__ tap,
                                                                 const float *__restrict__ dy,
                                                                 float *__restrict__ dx, PoolParams pp,
-                                                                int64_t total) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-    const int w = (int)(i % pp.W);
-    const int64_t t = i / pp.W;
-    const int h = (int)(t % pp.H);
-    const int64_t nc = t / pp.H;
+                                                                uint32_t total) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    uint32_t nc, pix, hh, ww;
+    pp.div_hw.divmod(i, nc, pix);
+    pp.div_w.divmod(pix, hh, ww);
+    const int h = (int)hh, w = (int)ww;
     // windows (p, q) with p*u - pad <= h <= p*u - pad + fh - 1
     const int p_lo = ceil_div_floor0(h + pp.pad_h - pp.fh + 1, pp.u);
     int p_hi = (h + pp.pad_h) / pp.u;
@@ -106,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned 
     const int q_lo = ceil_div_floor0(w + pp.pad_w - pp.fw + 1, pp.v);
     int q_hi = (w + pp.pad_w) / pp.v;
     if (q_hi > pp.Q - 1) q_hi = pp.Q - 1;
-    const int64_t win_base = nc * pp.P * pp.Q;
+    const int64_t win_base = (int64_t)nc * pp.P * pp.Q;
     float acc = 0.f;
     for (int p = p_lo; p <= p_hi; ++p) {
       const int r = h - (p * pp.u - pp.pad_h);
@@ -126,13 +131,15 @@ __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned 
 
 int grid_for(int64_t n) {
   int64_t blocks = (n + kThreads - 1) / kThreads;
-  const int64_t cap = (int64_t)num_cus() * 16;
+  const int64_t cap = (int64_t)num_cus() * 32;
   if (blocks > cap) blocks = cap;
   return blocks < 1 ? 1 : (int)blocks;
 }
 
 PoolParams params_of(const PoolDesc *d) {
-  return PoolParams{d->C, d->H, d->W, d->P, d->Q, d->pad_h, d->pad_w, d->u, d->v, d->fh, d->fw};
+  return PoolParams{d->C, d->H, d->W, d->P, d->Q, d->pad_h, d->pad_w, d->u, d->v, d->fh, d->fw,
+                    FastDiv((uint32_t)(d->P * d->Q)), FastDiv((uint32_t)d->Q), FastDiv((uint32_t)(d->H * d->W)),
+                    FastDiv((uint32_t)d->W)};
 }
 
 bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
@@ -188,13 +195,14 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
   hipStream_t s = stream_of(stream);
   const int64_t total = numel(output);
   if (total == 0) return 0;
+  TF_REQUIRE(numel(input) < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   const PoolParams pp = params_of(d);
   if (d->mode == 0)
     hipLaunchKernelGGL(pool_forward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s,
-                       (const float *)input->data, (float *)output->data, pp, total);
+                       (const float *)input->data, (float *)output->data, pp, (uint32_t)total);
   else
     hipLaunchKernelGGL(pool_forward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
-                       (const float *)input->data, (float *)output->data, pp, total);
+                       (const float *)input->data, (float *)output->data, pp, (uint32_t)total);
   return finish(s, "DLGpuPooling2DForward");
 }
 
@@ -212,6 +220,7 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
   hipStream_t s = stream_of(stream);
   const int64_t total = numel(dinput);
   if (total == 0) return 0;
+  TF_REQUIRE(total < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   const PoolParams pp = params_of(d);
   if (d->mode == 0) {
     TF_REQUIRE(d->fh * d->fw < 255, "max-pool windows of 255 or more taps are not supported");
@@ -219,14 +228,14 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
     unsigned char *tap = (unsigned char *)device_alloc((size_t)windows);
     TF_REQUIRE(tap, "out of device memory for %lld bytes of arg-max scratch", (long long)windows);
     hipLaunchKernelGGL(pool_argmax_kernel, dim3(grid_for(windows)), dim3(kThreads), 0, s,
-                       (const float *)input->data, tap, pp, windows);
+                       (const float *)input->data, tap, pp, (uint32_t)windows);
     hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
-                       (const float *)doutput->data, (float *)dinput->data, pp, total);
+                       (const float *)doutput->data, (float *)dinput->data, pp, (uint32_t)total);
     device_free(tap);  // stream-ordered reuse
   } else {
     hipLaunchKernelGGL(pool_backward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
                        (const unsigned char *)nullptr, (const float *)doutput->data, (float *)dinput->data, pp,
-                       total);
+                       (uint32_t)total);
   }
   return finish(s, "DLGpuPooling2DBackward");
 }
