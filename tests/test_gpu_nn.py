@@ -27,6 +27,11 @@ POOL_CASES = [
     ((3, 5, 13, 9), "max", 1, 0, 2, 1, 3, 2),
     ((3, 5, 13, 9), "mean", 1, 1, 2, 2, 3, 3),
     ((2, 3, 8, 8), "max", 0, 0, 1, 1, 1, 1),
+    ((2, 3, 11, 13), "max", 1, 1, 2, 2, 3, 3),      # odd extents: stride cells hang over the border
+    ((2, 3, 11, 13), "max", 0, 0, 3, 3, 3, 3),      # stride 3: per-element backward path
+    ((2, 3, 9, 10), "max", 1, 1, 1, 2, 3, 3),
+    ((2, 3, 9, 10), "max", 2, 2, 2, 1, 5, 4),
+    ((16, 64, 112, 112), "max", 1, 1, 2, 2, 3, 3),  # stem pool at full spatial size
 ]
 
 

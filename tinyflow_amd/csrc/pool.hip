@@ -129,6 +129,60 @@ __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned 
   }
 }
 
+// Max-pool backward, pass 2, for strides with u * v <= 4 (every configuration of
+// the reference models): one lane owns a u x v cell of dx aligned with the stride
+// grid.  The windows that can reach the cell are visited once each -- one tap byte
+// and at most one dy load per window -- instead of once per dx element, which cuts
+// the loads per element of dx by u * v.  The sum over windows runs in the same
+// (p, q) order as in the per-element kernel, so both give the same bits.
+__global__ __launch_bounds__(kThreads) void pool_backward_cell_kernel(const unsigned char *__restrict__ tap,
+                                                                     const float *__restrict__ dy,
+                                                                     float *__restrict__ dx, PoolParams pp,
+                                                                     FastDiv div_cells, FastDiv div_cw, int cells_h,
+                                                                     int cells_w, uint32_t total_cells) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total_cells; i += stride) {
+    uint32_t nc, cell, ci, cj;
+    div_cells.divmod(i, nc, cell);
+    div_cw.divmod(cell, ci, cj);
+    const int h0 = (int)ci * pp.u, w0 = (int)cj * pp.v;
+    const int p_lo = ceil_div_floor0(h0 + pp.pad_h - pp.fh + 1, pp.u);
+    int p_hi = (h0 + pp.u - 1 + pp.pad_h) / pp.u;
+    if (p_hi > pp.P - 1) p_hi = pp.P - 1;
+    const int q_lo = ceil_div_floor0(w0 + pp.pad_w - pp.fw + 1, pp.v);
+    int q_hi = (w0 + pp.v - 1 + pp.pad_w) / pp.v;
+    if (q_hi > pp.Q - 1) q_hi = pp.Q - 1;
+    const int64_t win_base = (int64_t)nc * pp.P * pp.Q;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int p = p_lo; p <= p_hi; ++p) {
+      for (int q = q_lo; q <= q_hi; ++q) {
+        const int64_t wi = win_base + p * pp.Q + q;
+        const int t = (int)tap[wi];
+        const int r = t / pp.fw, sft = t - r * pp.fw;
+        const int dh = p * pp.u - pp.pad_h + r - h0, dw = q * pp.v - pp.pad_w + sft - w0;
+        if (t != 255 && (unsigned)dh < (unsigned)pp.u && (unsigned)dw < (unsigned)pp.v) {
+          const float g = dy[wi];
+          const int slot = dh * pp.v + dw;
+          // register-resident accumulators: select instead of indexing
+          acc[0] += slot == 0 ? g : 0.f;
+          acc[1] += slot == 1 ? g : 0.f;
+          acc[2] += slot == 2 ? g : 0.f;
+          acc[3] += slot == 3 ? g : 0.f;
+        }
+      }
+    }
+    float *plane = dx + (int64_t)nc * pp.H * pp.W;
+    for (int dh = 0; dh < pp.u; ++dh)
+      for (int dw = 0; dw < pp.v; ++dw) {
+        const int h = h0 + dh, w = w0 + dw;
+        if (h < pp.H && w < pp.W) {
+          const int slot = dh * pp.v + dw;
+          plane[h * pp.W + w] = slot == 0 ? acc[0] : slot == 1 ? acc[1] : slot == 2 ? acc[2] : acc[3];
+        }
+      }
+  }
+}
+
 int grid_for(int64_t n) {
   int64_t blocks = (n + kThreads - 1) / kThreads;
   const int64_t cap = (int64_t)num_cus() * 32;
@@ -229,8 +283,17 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
     TF_REQUIRE(tap, "out of device memory for %lld bytes of arg-max scratch", (long long)windows);
     hipLaunchKernelGGL(pool_argmax_kernel, dim3(grid_for(windows)), dim3(kThreads), 0, s,
                        (const float *)input->data, tap, pp, (uint32_t)windows);
-    hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
-                       (const float *)doutput->data, (float *)dinput->data, pp, (uint32_t)total);
+    if (d->u * d->v <= 4) {
+      const int cells_h = cdiv(d->H, d->u), cells_w = cdiv(d->W, d->v);
+      const int64_t cells = (int64_t)d->N * d->C * cells_h * cells_w;
+      hipLaunchKernelGGL(pool_backward_cell_kernel, dim3(grid_for(cells)), dim3(kThreads), 0, s, tap,
+                         (const float *)doutput->data, (float *)dinput->data, pp,
+                         FastDiv((uint32_t)(cells_h * cells_w)), FastDiv((uint32_t)cells_w), cells_h, cells_w,
+                         (uint32_t)cells);
+    } else {
+      hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
+                         (const float *)doutput->data, (float *)dinput->data, pp, (uint32_t)total);
+    }
     device_free(tap);  // stream-ordered reuse
   } else {
     hipLaunchKernelGGL(pool_backward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
