@@ -73,21 +73,21 @@ def stream_handle(stream_cell):
 # commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
 # --config resnet50 --batch 64 only and are reported as null otherwise.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 133828328,
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 152173507,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 218982122,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 129468560,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 168480446,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 103308244,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 93419078,
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 92949775,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 198710998,
-    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 128625508,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 142659022,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126926815,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 160825147,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 139452498,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 104487652,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 133859676,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 152223946,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 219015322,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 129525365,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 168494569,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 103335109,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 93445590,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 92951163,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 198775724,
+    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 128693896,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 142682346,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126913095,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 160837791,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 139450426,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 104484332,
 }
 
 
