@@ -27,6 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBPS = 8000.0
 HBM_PEAK_GBS = 8000.0
 
 
@@ -145,18 +146,33 @@ class ConvTimer(object):
             return ret
         return timed
 
-    def pair_overhead_ms(self, stream, samples=32):
-        """Elapsed time an event pair reports with nothing between its two records
-        (median over a few pairs): subtracted from every kernel measurement."""
+    def pair_overhead_ms(self, stream, samples=24):
+        """What an event pair adds to the kernel it brackets: a small copy kernel is
+        launched `samples` times back to back inside one pair (per-launch time = the
+        bulk time / samples) and then once per pair; the difference of the two
+        per-launch times is subtracted from every kernel measurement."""
+        from tinyflow_amd import ndarray
+        src = ndarray.array(np.ones((4 << 20,), dtype=np.float32), ndarray.gpu(0))
+        dst = ndarray.empty((4 << 20,), ndarray.gpu(0))
+        cell = ctypes.cast(ctypes.pointer(ctypes.c_void_p(stream)), ctypes.POINTER(ctypes.c_void_p))
+        launch = lambda: self.gpu_op.matrix_elementwise_multiply_by_const(src, 1.0, dst, cell)
+        for _ in range(4):
+            launch()
+        e0, e1 = self._event(), self._event()
+        self.hip.record(e0, stream)
+        for _ in range(samples):
+            launch()
+        self.hip.record(e1, stream)
         pairs = [(self._event(), self._event()) for _ in range(samples)]
-        for e0, e1 in pairs:
-            self.hip.record(e0, stream)
-            self.hip.record(e1, stream)
+        for a, b in pairs:
+            self.hip.record(a, stream)
+            launch()
+            self.hip.record(b, stream)
         self.hip.sync()
-        vals = sorted(self.hip.elapsed_ms(e0, e1) for e0, e1 in pairs)
-        for e0, e1 in pairs:
-            self.pool += [e0, e1]
-        return vals[len(vals) // 2]
+        bulk = self.hip.elapsed_ms(e0, e1) / samples
+        single = sorted(self.hip.elapsed_ms(a, b) for a, b in pairs)[samples // 2]
+        self.pool += [e0, e1] + [e for pair in pairs for e in pair]
+        return max(single - bulk, 0.0)
 
     def collect(self, overhead_ms=0.0):
         """{variant: [launches, total_ms, total_flops]}; call after a device sync."""
@@ -170,6 +186,59 @@ class ConvTimer(object):
             self.pool += [e0, e1]
         self.pairs = []
         return stats
+
+
+class HbmTimer(object):
+    """HIP event pairs around the single-kernel, bandwidth-bound ops of a step
+    (batch norm, ReLU, residual add, max-pool backward, SGD) with the algorithmic
+    bytes each call moves, for the achieved-GB/s figures reported beside the
+    roofline of the dominant contraction kernel."""
+
+    def __init__(self, hip, gpu_op, pool, bn_mode):
+        self.hip, self.pool = hip, pool
+        self.enabled = False
+        self.pairs = []
+        n = lambda a: int(np.prod(a.shape))
+        bn_b = (8, 12) if bn_mode == "pre_activation" else (12, 20)
+        table = {
+            # op: bytes moved by one call, from its array arguments
+            "bn_forward": lambda a: bn_b[0] * n(a[0]),
+            "bn_backward": lambda a: bn_b[1] * n(a[0]),
+            "activation_forward": lambda a: 8 * n(a[0]),
+            "activation_backward": lambda a: 12 * n(a[0]),
+            "matrix_elementwise_add": lambda a: 12 * n(a[2]),
+            "pooling_2d_backward": lambda a: 4 * (n(a[0]) + n(a[1]) + n(a[2]) + n(a[3])),
+            "sgd_update": lambda a: 12 * n(a[0]),
+        }
+        for name, nbytes in table.items():
+            setattr(gpu_op, name, self._wrap(name, getattr(gpu_op, name), nbytes))
+
+    def _wrap(self, name, fn, nbytes):
+        def timed(*args):
+            if not self.enabled:
+                return fn(*args)
+            s = stream_handle(args[-1])
+            e0 = self.pool.pop() if self.pool else self.hip.event()
+            e1 = self.pool.pop() if self.pool else self.hip.event()
+            self.hip.record(e0, s)
+            ret = fn(*args)
+            self.hip.record(e1, s)
+            self.pairs.append((name, nbytes(args), e0, e1))
+            return ret
+        return timed
+
+    def collect(self, overhead_ms):
+        stats = {}
+        for name, nbytes, e0, e1 in self.pairs:
+            st = stats.setdefault(name, [0, 0.0, 0.0])
+            st[0] += 1
+            st[1] += max(self.hip.elapsed_ms(e0, e1) - overhead_ms, 1e-6)
+            st[2] += nbytes
+            self.pool += [e0, e1]
+        self.pairs = []
+        return [{"op": k, "launches": v[0], "avg_launch_us": v[1] / v[0] * 1e3, "bytes_per_launch": v[2] / v[0],
+                 "achieved_GBps": v[2] / (v[1] * 1e-3) / 1e9, "frac_of_hbm_peak": v[2] / (v[1] * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+                for k, v in sorted(stats.items(), key=lambda kv: -kv[1][1])]
 
 
 def cpu_baseline(bn_mode, sample_batch, image, repeats):
@@ -237,6 +306,7 @@ def main():
 
     hip = Hip()
     timer = ConvTimer(hip, gpu_op, _LIB)
+    hbm_timer = HbmTimer(hip, gpu_op, timer.pool, args.bn_mode)
     if args.batch is None:
         args.batch = {"mlp": 128, "lenet5": 64, "vgg16": 32, "resnet50": 64, "resnet152": 128}[args.config]
     kw = {"batch": args.batch}
@@ -294,6 +364,17 @@ def main():
     hip.sync()
     host_fed_ms = (time.perf_counter() - t1) * 1e3 / host_steps
 
+    # Bandwidth-bound kernels: two more steps (outside the timed region, their event
+    # pairs would weigh on `value`) with an event pair around each such call.
+    hbm_kernels = None
+    if not args.no_kernel_events:
+        hbm_timer.enabled = True
+        for _ in range(2):
+            ex.run(resident)
+        hbm_timer.enabled = False
+        hip.sync()
+        hbm_kernels = hbm_timer.collect(timer.pair_overhead_ms(s))
+
     if args.copy_calibration:
         from tinyflow_amd import ndarray
         src = ndarray.array(np.ones((64 << 20,), dtype=np.float32), ndarray.gpu(0))
@@ -341,6 +422,7 @@ def main():
         "host_fed": {"ms_per_step": host_fed_ms, "imgs_per_sec": args.batch * 1e3 / host_fed_ms, "steps": host_steps,
                      "note": "batch re-uploaded from pageable host memory every step (PCIe-inclusive)"},
         "roofline": roofline,
+        "hbm_kernels": hbm_kernels,
     }
     if swap_before:
         moved = {k: swap_after[k] - swap_before[k] for k in swap_after}
