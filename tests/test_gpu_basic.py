@@ -195,3 +195,44 @@ def test_copy_with_stream_and_d2d(rt):
     np.testing.assert_array_equal(host.asnumpy(), x)
     c = host.copyto(rt.ctx, rt.stream)
     np.testing.assert_array_equal(c.asnumpy(), x)
+
+
+def test_empty_tensors_are_accepted_everywhere(rt):
+    """Zero-element operands: every entry point returns success and launches nothing
+    (an empty batch, a layer with no outputs)."""
+    from tinyflow_amd import gpu_op, ndarray
+    e = lambda *shape: ndarray.empty(shape, rt.ctx)
+    a, b, c = e(0, 7), e(0, 7), e(0, 7)
+    gpu_op.array_set(a, 1.0, rt.stream)
+    gpu_op.matrix_elementwise_add(a, b, c, rt.stream)
+    gpu_op.matrix_elementwise_multiply(a, b, c, rt.stream)
+    gpu_op.matrix_elementwise_add_by_const(a, 2.0, c, rt.stream)
+    gpu_op.matrix_elementwise_multiply_by_const(a, 2.0, c, rt.stream)
+    gpu_op.relu(a, c)
+    gpu_op.relu_gradient(a, b, c)
+    gpu_op.softmax(a, c, rt.stream)
+    gpu_op.sgd_update(a, b, 0.1, rt.stream)
+    assert c.asnumpy().shape == (0, 7)
+    # matmul with an empty row set, and with an empty reduction (result is all zeros)
+    out = e(0, 5)
+    gpu_op.matrix_multiply(e(0, 7), False, e(7, 5), False, out, rt.cublas, rt.stream)
+    out = ndarray.array(np.full((3, 5), np.nan, np.float32), rt.ctx)
+    gpu_op.matrix_multiply(e(3, 0), False, e(0, 5), False, out, rt.cublas, rt.stream)
+    assert np.array_equal(out.asnumpy(), np.zeros((3, 5), np.float32))
+    # convolution, pooling, batch norm, activation on an empty batch
+    shape, wshape = (0, 3, 8, 8), (4, 3, 3, 3)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(shape, wshape, "NCHW", "SAME", 1, 1)
+    assert out_shape == (0, 4, 8, 8)
+    x, w, y = e(*shape), ndarray.array(np.ones(wshape, np.float32), rt.ctx), e(*out_shape)
+    dw = ndarray.array(np.full(wshape, np.nan, np.float32), rt.ctx)
+    assert gpu_op.convolution_2d_forward(x, w, y, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.convolution_backward_data(x, y, w, e(*shape), lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.convolution_backward_filter(x, y, w, dw, lst, rt.cudnn, rt.stream) == 0
+    assert np.array_equal(dw.asnumpy(), np.zeros(wshape, np.float32))   # empty reduction: zeros, not stale data
+    pshape, plst = gpu_op.pooling_2d_forward_get_out_shape(shape, "NCHW", "max", 0, 0, 2, 2, 2, 2)
+    py = e(*pshape)
+    gpu_op.pooling_2d_forward(x, py, plst, rt.cudnn, rt.stream)
+    gpu_op.pooling_2d_backward(x, py, py, e(*shape), plst, rt.cudnn, rt.stream)
+    alst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
+    gpu_op.activation_forward(x, e(*shape), "relu", alst, rt.cudnn, rt.stream)
+    gpu_op.activation_backward(x, e(*shape), x, x, "relu", alst, rt.cudnn, rt.stream)
