@@ -61,8 +61,10 @@ def multiply_by_const(a, c):
 
 
 def relu(x):
-    """reference autodiff.py:754 (np.maximum(x, 0)); gpu_op.cu:221-228"""
-    return np.maximum(x, 0)
+    """out = x, except 0 where x < 0: the CUDA kernel (gpu_op.cu:221-228), which
+    leaves a negative zero as it is.  The numpy branch (autodiff.py:754,
+    np.maximum(x, 0)) differs from it only in that sign of zero."""
+    return np.where(x < 0, np.zeros_like(x), x)
 
 
 def relu_gradient(x, grad):

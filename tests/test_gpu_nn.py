@@ -111,7 +111,7 @@ def test_activation(rt, shape, mode):
 
 
 BN_SHAPES = [(64, 64, 28, 28), (32, 16, 7, 9), (5, 3, 4, 4), (128, 8, 6, 6), (200, 4, 3, 3), (2, 2048, 7, 7),
-             (64, 1, 100)]
+             (64, 1, 100), (64, 256, 56, 56)]   # the last one: the largest ResNet-50 b64 activation
 
 
 @pytest.mark.parametrize("shape", BN_SHAPES, ids=str)
@@ -233,3 +233,27 @@ def test_dropout_and_concat_in_a_graph(rt):
     da1 = O.dropout_backward(dy1, keep, 0.4)
     np.testing.assert_allclose(grads[W1], X.T @ da1, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(grads[W2], X.T @ dy2, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_relu_masks_at_full_activation_size(rt):
+    """ReLU forward / backward on the largest ResNet-50 batch-64 activation
+    (64 x 256 x 56 x 56, 205 MB), through both entry-point families: bit-exact."""
+    from tinyflow_amd import gpu_op, ndarray
+    gen = np.random.default_rng(5)
+    shape = (64, 256, 56, 56)
+    x = gen.standard_normal(shape, dtype=np.float32)
+    x.reshape(-1)[::7] = 0.0          # exact zeros: the mask is x > 0
+    dy = gen.standard_normal(shape, dtype=np.float32)
+    want_y, want_dx = O.relu(x), O.relu_gradient(x, dy)
+    gx, gdy = ndarray.array(x, rt.ctx), ndarray.array(dy, rt.ctx)
+    gy, gdx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    gpu_op.relu(gx, gy)
+    gpu_op.relu_gradient(gx, gdy, gdx)
+    assert gy.asnumpy().tobytes() == want_y.tobytes() and gdx.asnumpy().tobytes() == want_dx.tobytes()
+    lst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
+    gpu_op.array_set(gy, np.nan, rt.stream)
+    gpu_op.array_set(gdx, np.nan, rt.stream)
+    gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+    gpu_op.activation_backward(gx, gdx, gy, gdy, "relu", lst, rt.cudnn, rt.stream)
+    assert gy.asnumpy().tobytes() == want_y.tobytes() and gdx.asnumpy().tobytes() == want_dx.tobytes()
