@@ -283,6 +283,10 @@ def main():
     ap.add_argument("--no-recompute", action="store_true",
                     help="with --mem-limit-gb: move every scheduled activation over PCIe instead of recomputing "
                          "batch-norm / ReLU outputs in the backward pass")
+    ap.add_argument("--fuse-bn-relu", action="store_true",
+                    help="run the timed steps with batch norm + ReLU evaluated as one kernel each way (an executor "
+                         "option outside the reference's op-by-op protocol; bit-identical results).  Without the "
+                         "flag the figure is still measured, on a second executor, and reported beside `value`")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--no-kernel-events", action="store_true",
@@ -320,7 +324,7 @@ def main():
         ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=int(0.95 * limit), prefetch_distance=12,
                           recompute=not args.no_recompute)
     else:
-        ex = TrainExecutor(model.loss, 0.01)
+        ex = TrainExecutor(model.loss, 0.01, fuse_bn_relu=args.fuse_bn_relu)
     ex.init_Variable(dict(model.variables))
     feed = {model.X: X, model.y_: y}
 
@@ -375,6 +379,29 @@ def main():
         hip.sync()
         hbm_kernels = hbm_timer.collect(timer.pair_overhead_ms(s))
 
+    # The same step with every batch norm + ReLU pair fused, on an executor of its own.
+    fused = None
+    if (not args.fuse_bn_relu and not args.mem_limit_gb and args.config.startswith("resnet")
+            and args.bn_mode == "pre_activation"):
+        model2, X2, y2 = models.build(args.config, **kw)
+        ex2 = TrainExecutor(model2.loss, 0.01, fuse_bn_relu=True)
+        ex2.init_Variable(dict(model2.variables))
+        ex2.run({model2.X: X2, model2.y_: y2})
+        for _ in range(2):
+            ex2.run({})
+        hip.sync()
+        fused_steps = max(2, min(args.steps, 10))
+        t2 = time.perf_counter()
+        for _ in range(fused_steps):
+            ex2.run({})
+        hip.sync()
+        fused_ms = (time.perf_counter() - t2) * 1e3 / fused_steps
+        fused = {"ms_per_step": fused_ms, "imgs_per_sec": args.batch * 1e3 / fused_ms, "steps": fused_steps,
+                 "fused_pairs": ex2.fused_pairs,
+                 "note": "batch norm + ReLU pairs evaluated by the fused entry points (executor option, not the "
+                         "reference's op-by-op protocol; results bit-identical)"}
+        del ex2, model2
+
     if args.copy_calibration:
         from tinyflow_amd import ndarray
         src = ndarray.array(np.ones((64 << 20,), dtype=np.float32), ndarray.gpu(0))
@@ -423,6 +450,7 @@ def main():
                      "note": "batch re-uploaded from pageable host memory every step (PCIe-inclusive)"},
         "roofline": roofline,
         "hbm_kernels": hbm_kernels,
+        "fused_bn_relu": fused,
     }
     if swap_before:
         moved = {k: swap_after[k] - swap_before[k] for k in swap_after}

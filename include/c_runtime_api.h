@@ -279,6 +279,20 @@ int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const DLArrayHand
                                     void **Variance_p, void ***list, void **handle,
                                     int *memorytoSaving, void **stream);
 
+/* No counterpart in the reference: batch norm and the ReLU that follows it as one
+ * pass (per-activation mode only).  Forward writes max(bn(x), 0); backward takes
+ * the gradient of that output and rebuilds the ReLU mask from x and the saved
+ * statistics.  Same arguments and statistics protocol as the plain pair above; the
+ * results equal those of the two separate ops bit for bit. */
+int DLGpuBatchNormalizationReluForward(const DLArrayHandle input, DLArrayHandle output,
+                                       int batchNormMode, int n, void **mean_p, void **Variance_p,
+                                       void ***list, void **handle, int *memorytoSaving,
+                                       void **stream);
+int DLGpuBatchNormalizationReluBackward(const DLArrayHandle input, const DLArrayHandle doutput,
+                                        DLArrayHandle dinput, int batchNormMode, void **mean_p,
+                                        void **Variance_p, void ***list, void **handle,
+                                        int *memorytoSaving, void **stream);
+
 /* ----------------------------------------------------- dropout, concatenation */
 
 /* Element-count descriptor that dropout takes in place of the reference's cuDNN

@@ -257,3 +257,54 @@ def test_relu_masks_at_full_activation_size(rt):
     gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
     gpu_op.activation_backward(gx, gdx, gy, gdy, "relu", lst, rt.cudnn, rt.stream)
     assert gy.asnumpy().tobytes() == want_y.tobytes() and gdx.asnumpy().tobytes() == want_dx.tobytes()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 64, 28, 28), (5, 3, 4, 4), (128, 8, 6, 6), (200, 4, 3, 3), (64, 256, 56, 56)],
+                         ids=str)
+def test_fused_batch_norm_relu_equals_the_two_ops(rt, shape):
+    """DLGpuBatchNormalizationRelu{Forward,Backward} against the separate batch-norm
+    and ReLU entry points: bit for bit, forward and backward."""
+    from tinyflow_amd import gpu_op, ndarray
+    gen = np.random.default_rng(8)
+    x = gen.standard_normal(shape, dtype=np.float32) * np.float32(1.7) + np.float32(0.3)
+    dy = gen.standard_normal(shape, dtype=np.float32)
+    gx, gdy = ndarray.array(x, rt.ctx), ndarray.array(dy, rt.ctx)
+    e = lambda: ndarray.empty(shape, rt.ctx)
+    # the two separate ops
+    mean_p, var_p, lst = gpu_op.bn_get_cudnnlist(shape, "NCHW", "pre_activation")
+    alst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
+    bn_out, relu_out, relu_dx, dx = e(), e(), e(), e()
+    assert gpu_op.bn_forward(gx, bn_out, "pre_activation", 0, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    gpu_op.activation_forward(bn_out, relu_out, "relu", alst, rt.cudnn, rt.stream)
+    gpu_op.activation_backward(bn_out, relu_dx, relu_out, gdy, "relu", alst, rt.cudnn, rt.stream)
+    assert gpu_op.bn_backward(gx, relu_dx, dx, "pre_activation", mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    # the fused pair
+    mean_p2, var_p2, lst2 = gpu_op.bn_get_cudnnlist(shape, "NCHW", "pre_activation")
+    fused_out, fused_dx = e(), e()
+    assert gpu_op.bn_relu_forward(gx, fused_out, "pre_activation", 0, mean_p2, var_p2, lst2, rt.cudnn, rt.stream) == 0
+    assert gpu_op.bn_relu_backward(gx, gdy, fused_dx, "pre_activation", mean_p2, var_p2, lst2, rt.cudnn,
+                                   rt.stream) == 0
+    assert fused_out.asnumpy().tobytes() == relu_out.asnumpy().tobytes()
+    assert fused_dx.asnumpy().tobytes() == dx.asnumpy().tobytes()
+    # and against the oracle's composition, within the batch-norm tolerance
+    if np.prod(shape) < 5_000_000:
+        x64 = x.astype(np.float64)
+        y_ref, mean, istd = O.batch_norm_forward(x64, "pre_activation")
+        np.testing.assert_allclose(fused_out.asnumpy(), np.maximum(y_ref, 0), rtol=1e-4, atol=1e-5)
+        dx_ref = O.batch_norm_backward(x64, np.where(y_ref > 0, dy.astype(np.float64), 0.0), "pre_activation", mean, istd)
+        got = fused_dx.asnumpy()
+        # elements whose normalised value is within rounding of 0 may fall on the other side of the mask
+        near = np.abs(y_ref) < 1e-5
+        if not near.any():
+            np.testing.assert_allclose(got, dx_ref, rtol=1e-3, atol=1e-5 * max(1.0, float(np.abs(dx_ref).max())))
+
+
+@pytest.mark.gpu
+def test_fused_batch_norm_relu_refuses_spatial_mode(rt):
+    from tinyflow_amd import gpu_op, ndarray
+    shape = (4, 3, 5, 5)
+    mean_p, var_p, lst = gpu_op.bn_get_cudnnlist(shape, "NCHW", "spatial")
+    x, y = ndarray.array(np.ones(shape, np.float32), rt.ctx), ndarray.empty(shape, rt.ctx)
+    with pytest.raises(RuntimeError):
+        gpu_op.bn_relu_forward(x, y, "spatial", 0, mean_p, var_p, lst, rt.cudnn, rt.stream)

@@ -134,3 +134,30 @@ def test_update_sees_forward_weights():
         if node.issgd:
             param = node.inputs[0]
             assert not any(param in later.inputs for later in order[i + 1:] if not later.issgd)
+
+
+@pytest.mark.gpu
+def test_fused_bn_relu_executor_is_bit_identical():
+    """TrainExecutor(fuse_bn_relu=True): same losses and parameters, bit for bit,
+    as the op-by-op executor over three steps; every conv-bn-relu triple is fused."""
+    from tinyflow_amd import models
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    runs = []
+    for fuse in (False, True):
+        rng = np.random.RandomState(21)
+        X, y = models.synthetic_batch(rng, (16, 3, 64, 64), 10, "normal")
+        model = models.resnet(rng, [2, 1, 1, 1], 16, image=64, n_class=10, bn_mode="pre_activation", width=8)
+        ex = TrainExecutor(model.loss, 0.01, fuse_bn_relu=fuse)
+        ex.init_Variable(dict(model.variables))
+        steps = []
+        for _ in range(3):
+            out = ex.run({model.X: X, model.y_: y})
+            steps.append([o.asnumpy() for o in out])
+        if fuse:
+            assert ex.fused_pairs == 1 + 2 * 5      # stem + two per bottleneck block
+        else:
+            assert ex.fused_pairs == 0
+        runs.append(steps)
+    for a_step, b_step in zip(*runs):
+        for a, b in zip(a_step, b_step):
+            assert a.tobytes() == b.tobytes()

@@ -20,7 +20,14 @@ from . import gpu_op, ndarray
 class TrainExecutor(object):
     """Runs forward + backward + SGD update for one loss node."""
 
-    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0)):
+    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), fuse_bn_relu=False):
+        """``fuse_bn_relu`` (no counterpart in the reference): evaluate every batch
+        norm whose only reader is a ReLU together with that ReLU, forward and
+        backward, through the fused entry points.  Results are bit-identical; the
+        batch-norm output and the ReLU's input gradient are then never materialised
+        (``value_of`` does not know them)."""
+        self.fuse_bn_relu = fuse_bn_relu
+        self.fused_pairs = 0
         self.targetloss = targetloss
         self.learning_rate = learning_rate
         self.Variable_node_list = ad.get_Variable_node_list(targetloss)
@@ -64,7 +71,19 @@ class TrainExecutor(object):
         feed_dict.update(self.Variable_node_np_value or {})
         self.infer_shape({node: np.shape(value) for node, value in feed_dict.items()})
         plan = []
+        fused = find_bn_relu_pairs(self.topo_order, {self.targetloss}) if self.fuse_bn_relu else {}
+        self.fused_pairs = sum(1 for v in fused.values() if v[0] == "forward")
         for node in self.topo_order:
+            role = fused.get(node)
+            if role is not None and role[0] == "skip":
+                continue   # its value is folded into the fused call of its reader
+            if role is not None:
+                kind, bn, sources = role
+                inputs = [self.node_to_arr_map[i] for i in sources]
+                node_val = self._alloc(self.node_to_shape_map[node])
+                self.node_to_arr_map[node] = node_val
+                plan.append((_fused_compute(kind, bn), node, inputs, node_val))
+                continue
             if node in feed_dict:
                 arr = ndarray.array(feed_dict[node], ctx=self.ctx)
                 if isinstance(arr, int):
@@ -107,6 +126,60 @@ class TrainExecutor(object):
     def value_of(self, node):
         """Device array currently holding ``node`` (any node of the step graph)."""
         return self.node_to_arr_map[node]
+
+
+def find_bn_relu_pairs(topo_order, outputs):
+    """Batch norms that can be evaluated together with the ReLU that follows them.
+
+    A per-activation batch-norm node B qualifies when its only readers are a ReLU
+    activation R and that activation's backward node A (which reads B as the ReLU
+    input), and A's only reader is B's own backward node D.  Returns a dict:
+    B and A -> ("skip",); R -> ("forward", B, [x]); D -> ("backward", B, [x, dR])."""
+    readers = {}
+    for n in topo_order:
+        for inp in n.inputs:
+            readers.setdefault(inp, []).append(n)
+    roles = {}
+    for r in topo_order:
+        if not (isinstance(r.op, ad.ActivationForwardOp) and r.activationMode == "relu"):
+            continue
+        b = r.inputs[0]
+        if not isinstance(b.op, ad.BNForwardOp) or b.batchNormMode != "pre_activation" or b in outputs:
+            continue
+        others = [n for n in readers.get(b, []) if n is not r]
+        if len(others) != 1:
+            continue
+        a = others[0]
+        if not (isinstance(a.op, ad.ActivationBackwardOp) and a.inputs[0] is b and a.inputs[2] is r) or a in outputs:
+            continue
+        a_readers = readers.get(a, [])
+        if len(a_readers) != 1:
+            continue
+        d = a_readers[0]
+        if not (isinstance(d.op, ad.BNBackwardOp) and d.inputs[1] is a and d.inputs[0] is b.inputs[0]
+                and d.Save_p is b.Save_p):
+            continue
+        roles[b] = ("skip",)
+        roles[a] = ("skip",)
+        roles[r] = ("forward", b, [b.inputs[0]])
+        roles[d] = ("backward", b, [b.inputs[0], a.inputs[1]])
+    return roles
+
+
+def _fused_compute(kind, bn):
+    """Plan entry (same signature as ``Op.compute``) that evaluates batch norm ``bn``
+    fused with its ReLU."""
+    if kind == "forward":
+        def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+            wanted = gpu_op.bn_relu_forward(input_vals[0], output_val, bn.batchNormMode, bn.n, bn.Save_p[0],
+                                            bn.Save_p[1], bn.cudnnlist[0], cudnnHandle, cudaStream)
+            bn.n += 1
+            return wanted
+    else:
+        def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+            return gpu_op.bn_relu_backward(input_vals[0], input_vals[1], output_val, bn.batchNormMode, bn.Save_p[0],
+                                           bn.Save_p[1], bn.cudnnlist[0], cudnnHandle, cudaStream)
+    return compute
 
 
 def getcomputelist(Variable_node_list, Variable_node_grad_list, learning_rate):

@@ -19,6 +19,8 @@
 // consumes and releases them.
 #include "internal.h"
 
+#include <type_traits>
+
 using namespace tf;
 
 namespace {
@@ -29,7 +31,8 @@ constexpr float kEps = 1e-5f;
 // ---------------------------------------------------------------- per-activation
 
 // NREG >= N values of one column live in registers.
-template <int NREG>
+// RELU: y = max(bn(x), 0) in the same pass (the fused entry points below).
+template <int NREG, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 float *__restrict__ save_mean,
@@ -54,10 +57,14 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   save_istd[l] = istd;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) y[(int64_t)n * L + l] = (v[n] - mean) * istd;
+    if (n < N) {
+      const float out = (v[n] - mean) * istd;
+      y[(int64_t)n * L + l] = (RELU && out < 0.f) ? 0.f : out;
+    }
 }
 
 // any N: three sweeps over the column (the second and third hit the cache)
+template <bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_forward_stream_kernel(const float *__restrict__ x,
                                                                        float *__restrict__ y,
                                                                        float *__restrict__ save_mean,
@@ -76,11 +83,15 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_stream_kernel(const fl
   const float istd = 1.0f / sqrtf(q / (float)N + kEps);
   save_mean[l] = mean;
   save_istd[l] = istd;
-  for (int n = 0; n < N; ++n) y[(int64_t)n * L + l] = (x[(int64_t)n * L + l] - mean) * istd;
+  for (int n = 0; n < N; ++n) {
+    const float out = (x[(int64_t)n * L + l] - mean) * istd;
+    y[(int64_t)n * L + l] = (RELU && out < 0.f) ? 0.f : out;
+  }
 }
 
 // dx = istd/N * (N*dy - sum(dy) - xhat * sum(dy*xhat))
-template <int NREG>
+// RELU: dy is first masked with bn(x) > 0, i.e. the gradient of max(bn(x), 0).
+template <int NREG, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *__restrict__ x,
                                                                  const float *__restrict__ dy,
                                                                  float *__restrict__ dx,
@@ -100,6 +111,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
 #pragma unroll
   for (int n = 0; n < NREG; ++n) {
     xh[n] = (xh[n] - mean) * istd;
+    if (RELU) g[n] = xh[n] > 0.f ? g[n] : 0.f;
     s1 += g[n];
     s2 += g[n] * xh[n];
   }
@@ -110,6 +122,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
     if (n < N) dx[(int64_t)n * L + l] = scale * (m * g[n] - s1 - xh[n] * s2);
 }
 
+template <bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_backward_stream_kernel(const float *__restrict__ x,
                                                                         const float *__restrict__ dy,
                                                                         float *__restrict__ dx,
@@ -121,15 +134,19 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_stream_kernel(const f
   const float mean = save_mean[l], istd = save_istd[l];
   float s1 = 0.f, s2 = 0.f;
   for (int n = 0; n < N; ++n) {
-    const float g = dy[(int64_t)n * L + l];
+    const float xh = (x[(int64_t)n * L + l] - mean) * istd;
+    float g = dy[(int64_t)n * L + l];
+    if (RELU) g = xh > 0.f ? g : 0.f;
     s1 += g;
-    s2 += g * ((x[(int64_t)n * L + l] - mean) * istd);
+    s2 += g * xh;
   }
   const float m = (float)N;
   const float scale = istd / m;
   for (int n = 0; n < N; ++n) {
     const float xh = (x[(int64_t)n * L + l] - mean) * istd;
-    dx[(int64_t)n * L + l] = scale * (m * dy[(int64_t)n * L + l] - s1 - xh * s2);
+    float g = dy[(int64_t)n * L + l];
+    if (RELU) g = xh > 0.f ? g : 0.f;
+    dx[(int64_t)n * L + l] = scale * (m * g - s1 - xh * s2);
   }
 }
 
@@ -292,16 +309,16 @@ extern "C" int DLGpuBatchNormalizationGetCudnnlist(const int *input_shapes, int 
   return 0;
 }
 
-extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArrayHandle output,
-                                              int batchNormMode, int n, void **mean_p, void **Variance_p,
-                                              void ***list, void **handle, int *memorytoSaving,
-                                              void **stream) {
+static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int batchNormMode, int n,
+                           void **mean_p, void **Variance_p, void ***list, void **handle, int *memorytoSaving,
+                           void **stream, bool relu, const char *what) {
   (void)handle;
   (void)n;  // would weight running statistics, which the reference never keeps
   BNDesc *d = desc_from_list<BNDesc>(list, kMagicBN);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuBatchNormalizationGetCudnnlist");
   TF_REQUIRE(d->mode == batchNormMode, "mode differs from the descriptor");
   TF_REQUIRE(mean_p && Variance_p, "null statistics cell");
+  TF_REQUIRE(!relu || d->mode == 0, "the fused batch-norm + ReLU entry points implement per-activation mode only");
   if (check_bn_arrays(d, input, output) != 0) return -1;
   hipStream_t s = stream_of(stream);
   const size_t stat_bytes = (size_t)d->stat_count * sizeof(float);
@@ -325,14 +342,18 @@ extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArray
   if (d->mode == 0) {
     const int64_t L = d->stat_count;
     const dim3 grid(cdiv(L, kThreads)), block(kThreads);
-    if (d->N <= 32)
-      hipLaunchKernelGGL(bn_pa_forward_kernel<32>, grid, block, 0, s, x, y, mean, istd, d->N, L);
-    else if (d->N <= 64)
-      hipLaunchKernelGGL(bn_pa_forward_kernel<64>, grid, block, 0, s, x, y, mean, istd, d->N, L);
-    else if (d->N <= 128)
-      hipLaunchKernelGGL(bn_pa_forward_kernel<128>, grid, block, 0, s, x, y, mean, istd, d->N, L);
-    else
-      hipLaunchKernelGGL(bn_pa_forward_stream_kernel, grid, block, 0, s, x, y, mean, istd, d->N, L);
+    auto run = [&](auto relu_c) {
+      constexpr bool RELU = decltype(relu_c)::value;
+      if (d->N <= 32)
+        hipLaunchKernelGGL((bn_pa_forward_kernel<32, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
+      else if (d->N <= 64)
+        hipLaunchKernelGGL((bn_pa_forward_kernel<64, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
+      else if (d->N <= 128)
+        hipLaunchKernelGGL((bn_pa_forward_kernel<128, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
+      else
+        hipLaunchKernelGGL(bn_pa_forward_stream_kernel<RELU>, grid, block, 0, s, x, y, mean, istd, d->N, L);
+    };
+    if (relu) run(std::true_type{}); else run(std::false_type{});
   } else {
     const int chunks = sp_chunks(d->N, d->C);
     const int ipc = cdiv(d->N, chunks);
@@ -354,13 +375,31 @@ extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArray
                        partial, mean, istd, d->N, d->C, d->HW, real_chunks);
     device_free(partial);
   }
-  return finish(s, "DLGpuBatchNormalizationForward");
+  return finish(s, what);
 }
 
-extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const DLArrayHandle doutput,
-                                               DLArrayHandle dinput, int batchNormMode, void **mean_p,
-                                               void **Variance_p, void ***list, void **handle,
-                                               int *memorytoSaving, void **stream) {
+extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArrayHandle output,
+                                              int batchNormMode, int n, void **mean_p, void **Variance_p,
+                                              void ***list, void **handle, int *memorytoSaving,
+                                              void **stream) {
+  return bn_forward_impl(input, output, batchNormMode, n, mean_p, Variance_p, list, handle, memorytoSaving, stream,
+                         false, "DLGpuBatchNormalizationForward");
+}
+
+// No counterpart in the reference: y = max(bn(x), 0) in one pass over x (8 bytes per
+// element instead of 16 for the two ops), per-activation mode.  Same statistics
+// protocol as the plain forward; pairs with DLGpuBatchNormalizationReluBackward.
+extern "C" int DLGpuBatchNormalizationReluForward(const DLArrayHandle input, DLArrayHandle output,
+                                                  int batchNormMode, int n, void **mean_p, void **Variance_p,
+                                                  void ***list, void **handle, int *memorytoSaving,
+                                                  void **stream) {
+  return bn_forward_impl(input, output, batchNormMode, n, mean_p, Variance_p, list, handle, memorytoSaving, stream,
+                         true, "DLGpuBatchNormalizationReluForward");
+}
+
+static int bn_backward_impl(const DLArrayHandle input, const DLArrayHandle doutput, DLArrayHandle dinput,
+                            int batchNormMode, void **mean_p, void **Variance_p, void ***list, void **handle,
+                            int *memorytoSaving, void **stream, bool relu, const char *what) {
   (void)handle;
   BNDesc *d = desc_from_list<BNDesc>(list, kMagicBN);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuBatchNormalizationGetCudnnlist");
@@ -370,6 +409,7 @@ extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const 
   TF_REQUIRE(mean_p && Variance_p && d->saved_mean && *mean_p == d->saved_mean &&
                  *Variance_p == d->saved_istd,
              "no saved statistics: backward needs the forward pass of the same step");
+  TF_REQUIRE(!relu || d->mode == 0, "the fused batch-norm + ReLU entry points implement per-activation mode only");
   if (check_bn_arrays(d, input, doutput) != 0) return -1;
   TF_REQUIRE(on_gpu(dinput) && numel(dinput) == numel(input), "dinput must have the input's shape");
   hipStream_t s = stream_of(stream);
@@ -380,14 +420,18 @@ extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const 
     if (d->mode == 0) {
       const int64_t L = d->stat_count;
       const dim3 grid(cdiv(L, kThreads)), block(kThreads);
-      if (d->N <= 32)
-        hipLaunchKernelGGL(bn_pa_backward_kernel<32>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
-      else if (d->N <= 64)
-        hipLaunchKernelGGL(bn_pa_backward_kernel<64>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
-      else if (d->N <= 128)
-        hipLaunchKernelGGL(bn_pa_backward_kernel<128>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
-      else
-        hipLaunchKernelGGL(bn_pa_backward_stream_kernel, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+      auto run = [&](auto relu_c) {
+        constexpr bool RELU = decltype(relu_c)::value;
+        if (d->N <= 32)
+          hipLaunchKernelGGL((bn_pa_backward_kernel<32, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+        else if (d->N <= 64)
+          hipLaunchKernelGGL((bn_pa_backward_kernel<64, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+        else if (d->N <= 128)
+          hipLaunchKernelGGL((bn_pa_backward_kernel<128, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+        else
+          hipLaunchKernelGGL(bn_pa_backward_stream_kernel<RELU>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+      };
+      if (relu) run(std::true_type{}); else run(std::false_type{});
     } else {
       const int chunks = sp_chunks(d->N, d->C);
       const int ipc = cdiv(d->N, chunks);
@@ -410,5 +454,25 @@ extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const 
   device_free(d->saved_istd);
   *mean_p = d->saved_mean = nullptr;
   *Variance_p = d->saved_istd = nullptr;
-  return finish(s, "DLGpuBatchNormalizationBackward");
+  return finish(s, what);
+}
+
+extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const DLArrayHandle doutput,
+                                               DLArrayHandle dinput, int batchNormMode, void **mean_p,
+                                               void **Variance_p, void ***list, void **handle,
+                                               int *memorytoSaving, void **stream) {
+  return bn_backward_impl(input, doutput, dinput, batchNormMode, mean_p, Variance_p, list, handle, memorytoSaving,
+                          stream, false, "DLGpuBatchNormalizationBackward");
+}
+
+// No counterpart in the reference: gradient of max(bn(x), 0) with respect to x.
+// doutput is the gradient of the ReLU output; the ReLU mask bn(x) > 0 is rebuilt
+// from x and the saved statistics, so neither bn(x) nor the ReLU output is read
+// (12 bytes per element instead of 24 for the two ops).
+extern "C" int DLGpuBatchNormalizationReluBackward(const DLArrayHandle input, const DLArrayHandle doutput,
+                                                   DLArrayHandle dinput, int batchNormMode, void **mean_p,
+                                                   void **Variance_p, void ***list, void **handle,
+                                                   int *memorytoSaving, void **stream) {
+  return bn_backward_impl(input, doutput, dinput, batchNormMode, mean_p, Variance_p, list, handle, memorytoSaving,
+                          stream, true, "DLGpuBatchNormalizationReluBackward");
 }

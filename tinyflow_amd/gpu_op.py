@@ -331,6 +331,29 @@ def bn_backward(input, doutput, dinput, batchNormMode, mean_p, var_p, cudnnlist,
     return wanted.value
 
 
+def bn_relu_forward(input, output, batchNormMode, n, mean_p, var_p, cudnnlist, cudnnHandle, cudaStream):
+    """max(bn(x), 0) in one pass (extension: no counterpart in the reference); same
+    arguments as ``bn_forward``."""
+    _nd_args(input, output)
+    mode = _enum(_BATCHNORM, batchNormMode)
+    wanted = ctypes.c_int(0)
+    check_call(_LIB.DLGpuBatchNormalizationReluForward(input.handle, output.handle, mode, n, mean_p, var_p,
+                                                       cudnnlist, cudnnHandle, ctypes.byref(wanted), cudaStream))
+    return wanted.value
+
+
+def bn_relu_backward(input, doutput, dinput, batchNormMode, mean_p, var_p, cudnnlist, cudnnHandle, cudaStream):
+    """Gradient of ``bn_relu_forward`` with respect to its input (extension); ``doutput``
+    is the gradient of the ReLU output."""
+    _nd_args(input, doutput, dinput)
+    mode = _enum(_BATCHNORM, batchNormMode)
+    wanted = ctypes.c_int(0)
+    check_call(_LIB.DLGpuBatchNormalizationReluBackward(input.handle, doutput.handle, dinput.handle, mode,
+                                                        mean_p, var_p, cudnnlist, cudnnHandle,
+                                                        ctypes.byref(wanted), cudaStream))
+    return wanted.value
+
+
 # ------------------------------------------------------------------- optimizers
 
 def sgd_update(output, g, learning_rate, cudaStream):
