@@ -128,6 +128,10 @@ int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB
                               DLArrayHandle output, void **stream);
 int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle input, float val,
                                      DLArrayHandle output, void **stream);
+/* No counterpart in the reference: output = max(matA + matB, 0), a residual join and
+ * the ReLU behind it as one pass; equals the two separate ops bit for bit. */
+int DLGpuMatrixElementwiseAddRelu(const DLArrayHandle matA, const DLArrayHandle matB,
+                                  DLArrayHandle output, void **stream);
 int DLGpuMatrixElementwiseMultiply(const DLArrayHandle matA, const DLArrayHandle matB,
                                    DLArrayHandle output, void **stream);
 int DLGpuMatrixMultiplyByConst(const DLArrayHandle input, float val,

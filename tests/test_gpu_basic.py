@@ -236,3 +236,19 @@ def test_empty_tensors_are_accepted_everywhere(rt):
     alst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
     gpu_op.activation_forward(x, e(*shape), "relu", alst, rt.cudnn, rt.stream)
     gpu_op.activation_backward(x, e(*shape), x, x, "relu", alst, rt.cudnn, rt.stream)
+
+
+@pytest.mark.parametrize("shape", [(64, 256, 28, 28), (5, 3), (1,), (1025,)])
+def test_add_relu_equals_add_then_relu(rt, shape):
+    from tinyflow_amd import gpu_op, ndarray
+    gen = np.random.default_rng(3)
+    a = gen.standard_normal(shape, dtype=np.float32)
+    b = gen.standard_normal(shape, dtype=np.float32)
+    b.reshape(-1)[::5] = -a.reshape(-1)[::5]      # exact zeros in the sum
+    ga, gb = ndarray.array(a, rt.ctx), ndarray.array(b, rt.ctx)
+    s, want, got = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    gpu_op.matrix_elementwise_add(ga, gb, s, rt.stream)
+    gpu_op.relu(s, want)
+    gpu_op.matrix_elementwise_add_relu(ga, gb, got, rt.stream)
+    assert got.asnumpy().tobytes() == want.asnumpy().tobytes()
+    assert got.asnumpy().tobytes() == O.relu(O.add(a, b)).tobytes()

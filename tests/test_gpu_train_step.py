@@ -154,7 +154,7 @@ def test_fused_bn_relu_executor_is_bit_identical():
             out = ex.run({model.X: X, model.y_: y})
             steps.append([o.asnumpy() for o in out])
         if fuse:
-            assert ex.fused_pairs == 1 + 2 * 5      # stem + two per bottleneck block
+            assert ex.fused_pairs == (1 + 2 * 5) + 5   # bn+relu: stem + two per block; add+relu: one per block
         else:
             assert ex.fused_pairs == 0
         runs.append(steps)

@@ -71,8 +71,11 @@ class TrainExecutor(object):
         feed_dict.update(self.Variable_node_np_value or {})
         self.infer_shape({node: np.shape(value) for node, value in feed_dict.items()})
         plan = []
-        fused = find_bn_relu_pairs(self.topo_order, {self.targetloss}) if self.fuse_bn_relu else {}
-        self.fused_pairs = sum(1 for v in fused.values() if v[0] == "forward")
+        fused = {}
+        if self.fuse_bn_relu:
+            fused.update(find_bn_relu_pairs(self.topo_order, {self.targetloss}))
+            fused.update(find_add_relu_pairs(self.topo_order, {self.targetloss}, self.node_to_shape_map))
+        self.fused_pairs = sum(1 for v in fused.values() if v[0] in ("forward", "add_relu"))
         for node in self.topo_order:
             role = fused.get(node)
             if role is not None and role[0] == "skip":
@@ -166,9 +169,51 @@ def find_bn_relu_pairs(topo_order, outputs):
     return roles
 
 
+def find_add_relu_pairs(topo_order, outputs, shapes):
+    """Elementwise sums that can be evaluated together with the ReLU that follows them
+    (the join of a residual block).  A sum S of two equally shaped values qualifies
+    when its only readers are a ReLU activation R and R's backward node A, which
+    reads S only to rebuild the mask S > 0 -- and R > 0 is the same mask.  Returns
+    S -> ("skip",); R -> ("add_relu", S, [a, b]); A -> ("mask_from_output", S, [R, dR, R])."""
+    readers = {}
+    for n in topo_order:
+        for inp in n.inputs:
+            readers.setdefault(inp, []).append(n)
+    roles = {}
+    for r in topo_order:
+        if not (isinstance(r.op, ad.ActivationForwardOp) and r.activationMode == "relu"):
+            continue
+        s = r.inputs[0]
+        if not isinstance(s.op, ad.AddOp) or s in outputs or len(s.inputs) != 2:
+            continue
+        if not (shapes[s.inputs[0]] == shapes[s.inputs[1]] == shapes[s]):
+            continue   # a (1,)-shaped operand is applied as a constant, not added elementwise
+        others = [n for n in readers.get(s, []) if n is not r]
+        if len(others) != 1:
+            continue
+        a = others[0]
+        if not (isinstance(a.op, ad.ActivationBackwardOp) and a.inputs[0] is s and a.inputs[2] is r):
+            continue
+        roles[s] = ("skip",)
+        roles[r] = ("add_relu", s, list(s.inputs))
+        roles[a] = ("mask_from_output", s, [r, a.inputs[1], r])
+    return roles
+
+
 def _fused_compute(kind, bn):
-    """Plan entry (same signature as ``Op.compute``) that evaluates batch norm ``bn``
-    fused with its ReLU."""
+    """Plan entry (same signature as ``Op.compute``) for a fused node: batch norm
+    ``bn`` with its ReLU (forward / backward), a sum with its ReLU, or a ReLU backward
+    that takes its mask from the ReLU output."""
+    if kind == "add_relu":
+        def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+            assert input_vals[0].shape == input_vals[1].shape == output_val.shape
+            gpu_op.matrix_elementwise_add_relu(input_vals[0], input_vals[1], output_val, cudaStream)
+            return 0
+        return compute
+    if kind == "mask_from_output":
+        def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+            return node.op.compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream)
+        return compute
     if kind == "forward":
         def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
             wanted = gpu_op.bn_relu_forward(input_vals[0], output_val, bn.batchNormMode, bn.n, bn.Save_p[0],

@@ -23,6 +23,8 @@ namespace {
 
 struct OpSet { float v; __device__ float operator()(float, float) const { return v; } };
 struct OpAdd { __device__ float operator()(float a, float b) const { return a + b; } };
+// max(a + b, 0): the sum keeps a negative zero, like the separate ReLU kernel does
+struct OpAddRelu { __device__ float operator()(float a, float b) const { const float t = a + b; return t < 0.f ? 0.f : t; } };
 struct OpMul { __device__ float operator()(float a, float b) const { return a * b; } };
 struct OpAddC { float v; __device__ float operator()(float a, float) const { return a + v; } };
 struct OpMulC { float v; __device__ float operator()(float a, float) const { return a * v; } };
@@ -122,6 +124,17 @@ extern "C" int DLGpuMatrixElementwiseAdd(const DLArrayHandle a, const DLArrayHan
   return launch_ew<OpAdd, true, true>(OpAdd{}, (float *)out->data, (const float *)a->data,
                                       (const float *)b->data, numel(out), stream_of(stream),
                                       "DLGpuMatrixElementwiseAdd");
+}
+
+// No counterpart in the reference: max(a + b, 0), the join of a residual block and
+// the ReLU that follows it, in one pass (12 bytes per element instead of 20).
+extern "C" int DLGpuMatrixElementwiseAddRelu(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
+                                             void **stream) {
+  TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
+  return launch_ew<OpAddRelu, true, true>(OpAddRelu{}, (float *)out->data, (const float *)a->data,
+                                          (const float *)b->data, numel(out), stream_of(stream),
+                                          "DLGpuMatrixElementwiseAddRelu");
 }
 
 extern "C" int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle in, float val, DLArrayHandle out,

@@ -106,6 +106,12 @@ def matrix_elementwise_add(matA, matB, matC, cudaStream):
     check_call(_LIB.DLGpuMatrixElementwiseAdd(matA.handle, matB.handle, matC.handle, cudaStream))
 
 
+def matrix_elementwise_add_relu(matA, matB, matC, cudaStream):
+    """max(matA + matB, 0) in one pass (extension: no counterpart in the reference)"""
+    _nd_args(matA, matB, matC)
+    check_call(_LIB.DLGpuMatrixElementwiseAddRelu(matA.handle, matB.handle, matC.handle, cudaStream))
+
+
 def matrix_elementwise_add_by_const(in_mat, val, out_mat, cudaStream):
     _nd_args(in_mat, out_mat)
     check_call(_LIB.DLGpuMatrixElementwiseAddByConst(in_mat.handle, ctypes.c_float(val),
