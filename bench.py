@@ -74,21 +74,21 @@ def stream_handle(stream_cell):
 # commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
 # --config resnet50 --batch 64 only and are reported as null otherwise.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 133859676,
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 152223946,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 219015322,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 129525365,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 168494569,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 103335109,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 93445590,
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 92951163,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 198775724,
-    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 128693896,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 142682346,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126913095,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 160837791,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 139450426,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 104484332,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 917379966,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 812899912,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 424364956,
+    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 634931576,
+    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 633969815,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 618614572,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 1153202304,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 516559950,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 340282125,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 840789188,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 474898113,
+    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 337306987,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 346140388,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 505250803,
+    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 282734170,
 }
 
 
