@@ -84,6 +84,32 @@ def test_max_pool_routing_is_first_maximum(rt):
     np.testing.assert_array_equal(gdx.asnumpy()[0, 0], expect)
 
 
+@pytest.mark.parametrize("case", [((4, 8, 28, 28), 1, 1, 2, 2, 3, 3), ((2, 3, 11, 13), 0, 0, 3, 3, 3, 3)],
+                         ids=["overlapping", "stride3"])
+def test_max_pool_backward_without_scratch_memory(rt, case):
+    """With no device memory left for the arg-max scratch the backward pass still
+    runs (the entry point cannot report out-of-memory) and gives the same bits."""
+    from tinyflow_amd import gpu_op, ndarray
+    shape, ph, pw, u, v, fh, fw = case
+    rng = np.random.RandomState(23)
+    x = np.maximum(np.round(rng.normal(0, 1, shape) * 2) / 2, 0).astype(np.float32)
+    out_shape, lst = gpu_op.pooling_2d_forward_get_out_shape(shape, "NCHW", "max", ph, pw, u, v, fh, fw)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx, gdx2 = ndarray.empty(out_shape, rt.ctx), ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    gpu_op.pooling_2d_forward(gx, gy, lst, rt.cudnn, rt.stream)
+    gpu_op.pooling_2d_backward(gx, gy, gdy, gdx, lst, rt.cudnn, rt.stream)
+    _, in_use, _ = gpu_op.device_memory_stats()
+    gpu_op.set_device_memory_limit(max(in_use, 1))   # nothing more can be allocated
+    try:
+        assert isinstance(ndarray.empty((1 << 20,), rt.ctx), int)   # the budget really is exhausted
+        gpu_op.pooling_2d_backward(gx, gy, gdy, gdx2, lst, rt.cudnn, rt.stream)
+        got = gdx2.asnumpy()
+    finally:
+        gpu_op.set_device_memory_limit(0)
+    np.testing.assert_array_equal(got, gdx.asnumpy())
+
+
 @pytest.mark.parametrize("shape", [(64, 256, 14, 14), (3, 5, 7, 9), (128, 100), (7, 1, 33)])
 @pytest.mark.parametrize("mode", ["relu", "sigmoid", "tanh", "softmax"])
 def test_activation(rt, shape, mode):

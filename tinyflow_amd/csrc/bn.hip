@@ -292,14 +292,17 @@ extern "C" int DLGpuBatchNormalizationGetCudnnlist(const int *input_shapes, int 
   TF_REQUIRE(sizeofshape >= 2 && sizeofshape <= 5, "rank %d not supported", sizeofshape);
   TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
   TF_REQUIRE(batchNormMode == 0 || batchNormMode == 1, "unknown batch-norm mode %d", batchNormMode);
+  int64_t hw = 1;
+  for (int i = 0; i < sizeofshape; ++i) {
+    TF_REQUIRE(input_shapes[i] >= 0, "negative extent");
+    if (i >= 2) hw *= input_shapes[i];
+    TF_REQUIRE(hw <= INT32_MAX, "spatial extent too large");
+  }
   BNDesc *d = new BNDesc();
   d->magic = kMagicBN;
   d->mode = batchNormMode;
   d->N = input_shapes[0];
   d->C = input_shapes[1];
-  int64_t hw = 1;
-  for (int i = 2; i < sizeofshape; ++i) hw *= input_shapes[i];
-  TF_REQUIRE(hw <= INT32_MAX, "spatial extent too large");
   d->HW = (int)hw;
   d->stat_count = batchNormMode == 0 ? (int64_t)d->C * d->HW : d->C;
   d->saved_mean = d->saved_istd = nullptr;
@@ -331,7 +334,7 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
   float *istd = mean ? (float *)device_alloc(stat_bytes) : nullptr;
   if (!mean || !istd) {
     if (mean) device_free(mean);
-    if (memorytoSaving) *memorytoSaving = (int)stat_bytes;
+    if (memorytoSaving) *memorytoSaving = shortfall(stat_bytes);
     return 0;
   }
   *mean_p = d->saved_mean = mean;
@@ -365,7 +368,7 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
       device_free(istd);
       *mean_p = d->saved_mean = nullptr;
       *Variance_p = d->saved_istd = nullptr;
-      if (memorytoSaving) *memorytoSaving = (int)pbytes;
+      if (memorytoSaving) *memorytoSaving = shortfall(pbytes);
       return 0;
     }
     hipLaunchKernelGGL(bn_sp_partial_kernel<false>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x,
@@ -439,7 +442,7 @@ static int bn_backward_impl(const DLArrayHandle input, const DLArrayHandle doutp
       const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double);
       double *partial = (double *)device_alloc(pbytes);
       if (!partial) {
-        if (memorytoSaving) *memorytoSaving = (int)pbytes;
+        if (memorytoSaving) *memorytoSaving = shortfall(pbytes);
         return 0;  // statistics stay published so the call can be repeated
       }
       hipLaunchKernelGGL(bn_sp_partial_kernel<true>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x, dy,

@@ -524,7 +524,14 @@ extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, con
   TF_REQUIRE(input_shapes && filter_shapes && output_shapes && list, "null argument");
   TF_REQUIRE(dataformat == 0, "only NCHW (dataformat 0) is implemented");
   TF_REQUIRE(u >= 1 && v >= 1, "strides must be positive");
-  ConvDesc *d = new ConvDesc();
+  for (int i = 0; i < 4; ++i)
+    TF_REQUIRE(input_shapes[i] >= 0 && filter_shapes[i] >= 0, "negative extent");
+  TF_REQUIRE(filter_shapes[1] == input_shapes[1], "filter expects %d input channels, input has %d",
+             filter_shapes[1], input_shapes[1]);
+  TF_REQUIRE(filter_shapes[2] >= 1 && filter_shapes[3] >= 1 && filter_shapes[2] <= 32 && filter_shapes[3] <= 32,
+             "filter extents must lie in 1..32");
+  ConvDesc desc;
+  ConvDesc *d = &desc;
   d->magic = kMagicConv;
   d->N = input_shapes[0];
   d->C = input_shapes[1];
@@ -533,7 +540,6 @@ extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, con
   d->K = filter_shapes[0];
   d->R = filter_shapes[2];
   d->S = filter_shapes[3];
-  TF_REQUIRE(filter_shapes[1] == d->C, "filter expects %d input channels, input has %d", filter_shapes[1], d->C);
   d->pad_h = padding == 1 ? d->R / 2 : 0;  // "SAME" is a symmetric k/2, "VALID" is 0
   d->pad_w = padding == 1 ? d->S / 2 : 0;
   d->u = u;
@@ -541,7 +547,7 @@ extern "C" int DLGpuConvolution2DForwardGetOutShape(const int *input_shapes, con
   TF_REQUIRE(d->H + 2 * d->pad_h >= d->R && d->W + 2 * d->pad_w >= d->S, "filter larger than padded input");
   d->P = 1 + (d->H + 2 * d->pad_h - d->R) / u;
   d->Q = 1 + (d->W + 2 * d->pad_w - d->S) / v;
-  TF_REQUIRE(d->R <= 32 && d->S <= 32, "filter extents above 32 are not supported");
+  d = new ConvDesc(desc);
   output_shapes[0] = d->N;
   output_shapes[1] = d->K;
   output_shapes[2] = d->P;
@@ -574,6 +580,7 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
   const ConvPlan plan = plan_forward(d);
   const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
+  if (K == 0) return DLGpuArraySet(output, 0.f, stream);
   const int bm = plan.bm, bn = plan.bn;
   const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
   float *partial = nullptr;
@@ -581,7 +588,7 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
     const size_t bytes = (size_t)g.splits * numel(output) * sizeof(float);
     partial = (float *)device_alloc(bytes);
     if (!partial) {
-      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
   }
@@ -631,7 +638,7 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     const size_t bytes = (size_t)numel(filter) * sizeof(float);
     wt_scratch = (float *)device_alloc(bytes);
     if (!wt_scratch) {
-      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
     const int total = (int)numel(filter);
@@ -647,7 +654,7 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     partial = (float *)device_alloc(bytes);
     if (!partial) {
       if (wt_scratch) device_free(wt_scratch);
-      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
   }
@@ -733,7 +740,7 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
     const size_t bytes = (size_t)g.splits * M * N * sizeof(float);
     partial = (float *)device_alloc(bytes);
     if (!partial) {
-      if (memorytoSaving) *memorytoSaving = (int)bytes;
+      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
     dst = partial;

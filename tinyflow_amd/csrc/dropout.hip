@@ -173,7 +173,7 @@ extern "C" int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle outp
   const int64_t groups = (in->count + 7) / 8;
   unsigned char *mask = (unsigned char *)device_alloc((size_t)(groups > 0 ? groups : 1));
   if (!mask) {
-    if (memorytoSaving) *memorytoSaving = (int)groups;
+    if (memorytoSaving) *memorytoSaving = shortfall(groups);
     return 0;
   }
   DropoutDesc *d = new DropoutDesc();

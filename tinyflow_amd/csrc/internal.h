@@ -41,6 +41,15 @@ inline bool on_gpu(const DLArray *a) { return a && a->data && a->ctx.device_type
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
+// Value stored through `memorytoSaving` when an allocation of `bytes` fails.  The
+// caller reads "non-zero" as "out of memory, this much was wanted"
+// (src/c_runtime_api.cc:109-113 casts the size to int); the cast is saturated here
+// so that a request of 2 GiB or more can neither wrap to zero nor go negative.
+inline int shortfall(size_t bytes) {
+  if (bytes == 0) return 1;
+  return bytes > (size_t)0x7fffffff ? 0x7fffffff : (int)bytes;
+}
+
 // Number of compute units of the current device (256 on MI355X).
 int num_cus();
 

@@ -60,8 +60,29 @@ __device__ inline int ceil_div_floor0(int a, int b) {  // ceil(a / b) clamped at
   return a <= 0 ? 0 : (a + b - 1) / b;
 }
 
-// Max-pool backward, pass 1: one lane per window records which tap (r * fw + s)
-// holds the window's first maximum in row-major order.
+// Tap (r * fw + s) that holds the first maximum of window (p, q) of `plane` in
+// row-major order; 255 when the window holds no comparable value (all NaN).
+__device__ inline int window_argmax(const float *__restrict__ plane, const PoolParams &pp, int p, int q) {
+  const int h0 = p * pp.u - pp.pad_h, w0 = q * pp.v - pp.pad_w;
+  float best = -INFINITY;
+  int arg = 255;
+  for (int r = 0; r < pp.fh; ++r) {
+    const int h = h0 + r;
+    if ((unsigned)h >= (unsigned)pp.H) continue;
+    for (int s = 0; s < pp.fw; ++s) {
+      const int w = w0 + s;
+      if ((unsigned)w >= (unsigned)pp.W) continue;
+      const float val = plane[h * pp.W + w];
+      if (val > best || (arg == 255 && val == best)) {  // strict: the first maximum wins
+        best = val;
+        arg = r * pp.fw + s;
+      }
+    }
+  }
+  return arg;
+}
+
+// Max-pool backward, pass 1: one lane per window records the window's arg-max tap.
 __global__ __launch_bounds__(kThreads) void pool_argmax_kernel(const float *__restrict__ x,
                                                               unsigned char *__restrict__ tap, PoolParams pp,
                                                               uint32_t total) {
@@ -70,31 +91,17 @@ __global__ __launch_bounds__(kThreads) void pool_argmax_kernel(const float *__re
     uint32_t nc, pix, p, q;
     pp.div_pq.divmod(i, nc, pix);
     pp.div_q.divmod(pix, p, q);
-    const int h0 = (int)p * pp.u - pp.pad_h, w0 = (int)q * pp.v - pp.pad_w;
-    const float *plane = x + (int64_t)nc * pp.H * pp.W;
-    float best = -INFINITY;
-    int arg = 255;  // stays 255 when the window holds no comparable value (all NaN)
-    for (int r = 0; r < pp.fh; ++r) {
-      const int h = h0 + r;
-      if ((unsigned)h >= (unsigned)pp.H) continue;
-      for (int s = 0; s < pp.fw; ++s) {
-        const int w = w0 + s;
-        if ((unsigned)w >= (unsigned)pp.W) continue;
-        const float val = plane[h * pp.W + w];
-        if (val > best || (arg == 255 && val == best)) {  // strict: the first maximum wins
-          best = val;
-          arg = r * pp.fw + s;
-        }
-      }
-    }
-    tap[i] = (unsigned char)arg;
+    tap[i] = (unsigned char)window_argmax(x + (int64_t)nc * pp.H * pp.W, pp, (int)p, (int)q);
   }
 }
 
 // Pass 2 (max) / the whole backward (mean): one lane per INPUT pixel gathers dy
-// from the windows that cover it.
+// from the windows that cover it.  With MAX and no tap array (the scratch for it
+// could not be allocated) every covering window's arg-max is recomputed from x:
+// slower, same bits, no memory beyond the operands.
 template <bool MAX>
 __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned char *__restrict__ tap,
+                                                                const float *__restrict__ x,
                                                                 const float *__restrict__ dy,
                                                                 float *__restrict__ dx, PoolParams pp,
                                                                 uint32_t total) {
@@ -119,7 +126,8 @@ __global__ __launch_bounds__(kThreads) void pool_backward_kernel(const unsigned 
         const int64_t wi = win_base + p * pp.Q + q;
         if (MAX) {
           const int s = w - (q * pp.v - pp.pad_w);
-          if ((int)tap[wi] == r * pp.fw + s) acc += dy[wi];
+          const int t = tap ? (int)tap[wi] : window_argmax(x + (int64_t)nc * pp.H * pp.W, pp, p, q);
+          if (t == r * pp.fw + s) acc += dy[wi];
         } else {
           acc += dy[wi];
         }
@@ -211,6 +219,9 @@ extern "C" int DLGpuPooling2DForwardGetOutShape(const int *input_shapes, int *ou
   TF_REQUIRE(poolingMode == 0 || poolingMode == 1, "unknown pooling mode %d", poolingMode);
   TF_REQUIRE(u >= 1 && v >= 1 && filter_h >= 1 && filter_w >= 1 && padding_h >= 0 && padding_w >= 0,
              "bad window geometry");
+  for (int i = 0; i < 4; ++i) TF_REQUIRE(input_shapes[i] >= 0, "negative extent");
+  TF_REQUIRE(input_shapes[2] + 2 * padding_h >= filter_h && input_shapes[3] + 2 * padding_w >= filter_w,
+             "window larger than padded input");
   PoolDesc *d = new PoolDesc();
   d->magic = kMagicPool;
   d->N = input_shapes[0];
@@ -224,8 +235,6 @@ extern "C" int DLGpuPooling2DForwardGetOutShape(const int *input_shapes, int *ou
   d->v = v;
   d->fh = filter_h;
   d->fw = filter_w;
-  TF_REQUIRE(d->H + 2 * padding_h >= filter_h && d->W + 2 * padding_w >= filter_w,
-             "window larger than padded input");
   d->P = 1 + (d->H + 2 * padding_h - filter_h) / u;
   d->Q = 1 + (d->W + 2 * padding_w - filter_w) / v;
   output_shapes[0] = d->N;
@@ -279,11 +288,13 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
   if (d->mode == 0) {
     TF_REQUIRE(d->fh * d->fw < 255, "max-pool windows of 255 or more taps are not supported");
     const int64_t windows = numel(doutput);
+    // this entry point has no way to report a failed allocation to the caller
+    // (no memorytoSaving argument), so it must also work without the scratch
     unsigned char *tap = (unsigned char *)device_alloc((size_t)windows);
-    TF_REQUIRE(tap, "out of device memory for %lld bytes of arg-max scratch", (long long)windows);
-    hipLaunchKernelGGL(pool_argmax_kernel, dim3(grid_for(windows)), dim3(kThreads), 0, s,
-                       (const float *)input->data, tap, pp, (uint32_t)windows);
-    if (d->u * d->v <= 4) {
+    if (tap)
+      hipLaunchKernelGGL(pool_argmax_kernel, dim3(grid_for(windows)), dim3(kThreads), 0, s,
+                         (const float *)input->data, tap, pp, (uint32_t)windows);
+    if (tap && d->u * d->v <= 4) {
       const int cells_h = cdiv(d->H, d->u), cells_w = cdiv(d->W, d->v);
       const int64_t cells = (int64_t)d->N * d->C * cells_h * cells_w;
       hipLaunchKernelGGL(pool_backward_cell_kernel, dim3(grid_for(cells)), dim3(kThreads), 0, s, tap,
@@ -292,13 +303,14 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
                          (uint32_t)cells);
     } else {
       hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
-                         (const float *)doutput->data, (float *)dinput->data, pp, (uint32_t)total);
+                         (const float *)input->data, (const float *)doutput->data, (float *)dinput->data, pp,
+                         (uint32_t)total);
     }
-    device_free(tap);  // stream-ordered reuse
+    if (tap) device_free(tap);  // stream-ordered reuse
   } else {
     hipLaunchKernelGGL(pool_backward_kernel<false>, dim3(grid_for(total)), dim3(kThreads), 0, s,
-                       (const unsigned char *)nullptr, (const float *)doutput->data, (float *)dinput->data, pp,
-                       (uint32_t)total);
+                       (const unsigned char *)nullptr, (const float *)nullptr, (const float *)doutput->data,
+                       (float *)dinput->data, pp, (uint32_t)total);
   }
   return finish(s, "DLGpuPooling2DBackward");
 }

@@ -179,10 +179,17 @@ __global__ __launch_bounds__(kThreads) void zero_kernel(float *out, int n) {
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // out[b] = sum_{a, c} in[a, b, c]; 0 on success, 1 when scratch is exhausted
-// (then *scratch_bytes holds the size wanted), -1 on launch failure.
+// (then *scratch_bytes holds the size wanted), -1 on launch failure.  A caller
+// that cannot report exhausted scratch passes scratch_bytes == nullptr: the sum
+// then runs as a single chunk, which needs no scratch (slower on short outputs,
+// and the additions associate differently than in the chunked run).
 int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hipStream_t s,
                size_t *scratch_bytes, const char *what) {
   if (B == 0) return 0;
+  if (A > INT32_MAX || B > INT32_MAX || C > INT32_MAX) {
+    fprintf(stderr, "[tinyflow_amd] %s: extents of 2^31 or more are not supported\n", what);
+    return -1;
+  }
   if (A == 0 || C == 0) {  // empty sum: a fill kernel, which (unlike a memset node) is safe under graph capture
     hipLaunchKernelGGL(zero_kernel, dim3(cdiv(B, kThreads)), dim3(kThreads), 0, s, out, (int)B);
     return finish(s, what);
@@ -197,15 +204,20 @@ int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hip
     if (chunks > max_chunks) chunks = (int)max_chunks;
     if (chunks < 1) chunks = 1;
   }
-  const int rows_per_chunk = (int)((A + chunks - 1) / chunks);
+  int rows_per_chunk = (int)((A + chunks - 1) / chunks);
   chunks = (int)((A + rows_per_chunk - 1) / rows_per_chunk);
   float *partial = out;
   if (chunks > 1) {
     const size_t bytes = (size_t)chunks * (size_t)B * sizeof(float);
     partial = (float *)device_alloc(bytes);
     if (!partial) {
-      *scratch_bytes = bytes;
-      return 1;
+      if (scratch_bytes) {
+        *scratch_bytes = bytes;
+        return 1;
+      }
+      partial = out;
+      chunks = 1;
+      rows_per_chunk = (int)A;
     }
   }
   if (C == 1) {
@@ -234,14 +246,9 @@ extern "C" int DLGpuReduceSumAxisZero(const DLArrayHandle in, DLArrayHandle out)
   const int64_t A = in->shape[0];
   const int64_t B = numel(in) / (A > 0 ? A : 1);
   TF_REQUIRE(numel(out) == (in->ndim == 1 ? 1 : B), "output must be input.shape[1:]");
-  size_t want = 0;
   // 1-D input (n,) -> (1,): one column of n rows
-  const int rc = in->ndim == 1 ? reduce_abc((const float *)in->data, (float *)out->data, A, 1, 1, nullptr,
-                                            &want, "DLGpuReduceSumAxisZero")
-                               : reduce_abc((const float *)in->data, (float *)out->data, A, B, 1, nullptr,
-                                            &want, "DLGpuReduceSumAxisZero");
-  TF_REQUIRE(rc == 0, "failed (scratch bytes wanted: %zu)", want);
-  return 0;
+  return reduce_abc((const float *)in->data, (float *)out->data, A, in->ndim == 1 ? 1 : B, 1, nullptr, nullptr,
+                    "DLGpuReduceSumAxisZero");
 }
 
 extern "C" int DLGpuBroadcastToBackward0(const DLArrayHandle in, DLArrayHandle out) {
@@ -254,11 +261,8 @@ extern "C" int DLGpuBroadcastToBackward0(const DLArrayHandle in, DLArrayHandle o
       TF_REQUIRE(in->shape[in->ndim - 1 - i] == out->shape[out->ndim - 1 - i],
                  "output must match the trailing dims of the input");
   }
-  size_t want = 0;
-  const int rc = reduce_abc((const float *)in->data, (float *)out->data, numel(in) / B, B, 1, nullptr, &want,
-                            "DLGpuBroadcastToBackward0");
-  TF_REQUIRE(rc == 0, "failed (scratch bytes wanted: %zu)", want);
-  return 0;
+  return reduce_abc((const float *)in->data, (float *)out->data, numel(in) / B, B, 1, nullptr, nullptr,
+                    "DLGpuBroadcastToBackward0");
 }
 
 extern "C" int DLGpuBroadcastToBackward1(const DLArrayHandle in, DLArrayHandle out) {
@@ -267,11 +271,8 @@ extern "C" int DLGpuBroadcastToBackward1(const DLArrayHandle in, DLArrayHandle o
              "input must be (N, C, ...) and output (C,)");
   int64_t inner = 1;
   for (int i = 2; i < in->ndim; ++i) inner *= in->shape[i];
-  size_t want = 0;
-  const int rc = reduce_abc((const float *)in->data, (float *)out->data, in->shape[0], in->shape[1], inner,
-                            nullptr, &want, "DLGpuBroadcastToBackward1");
-  TF_REQUIRE(rc == 0, "failed (scratch bytes wanted: %zu)", want);
-  return 0;
+  return reduce_abc((const float *)in->data, (float *)out->data, in->shape[0], in->shape[1], inner, nullptr,
+                    nullptr, "DLGpuBroadcastToBackward1");
 }
 
 extern "C" int DLGReduceSumGetCudnnlist(const int *input_shapes, const int *output_shapes, const int ndim,
@@ -280,13 +281,15 @@ extern "C" int DLGReduceSumGetCudnnlist(const int *input_shapes, const int *outp
   (void)handle;
   TF_REQUIRE(input_shapes && output_shapes && list, "null argument");
   TF_REQUIRE(ndim >= 1 && ndim <= 5, "rank %d not supported", ndim);
+  for (int i = 0; i < ndim; ++i)
+    TF_REQUIRE(input_shapes[i] >= 0 && (output_shapes[i] == input_shapes[i] || output_shapes[i] == 1),
+               "output dim %d must be 1 or equal to the input dim", i);
   ReduceDesc *d = new ReduceDesc();
   d->magic = kMagicReduce;
   d->ndim = ndim;
   for (int i = 0; i < ndim; ++i) {
     d->in[i] = input_shapes[i];
     d->out[i] = output_shapes[i];
-    TF_REQUIRE(d->out[i] == d->in[i] || d->out[i] == 1, "output dim %d must be 1 or equal to the input dim", i);
   }
   // same five-slot list as the reference; every slot points at the descriptor
   void **slots = (void **)malloc(sizeof(void *) * 5);
@@ -329,7 +332,7 @@ extern "C" int DLGpuReduceSum(const DLArrayHandle in, DLArrayHandle out, void **
   const int rc = reduce_abc((const float *)in->data, (float *)out->data, A, B, C, stream_of(stream), &want,
                             "DLGpuReduceSum");
   if (rc == 1) {
-    if (memorytoSaving) *memorytoSaving = (int)want;
+    if (memorytoSaving) *memorytoSaving = shortfall(want);
     return 0;
   }
   return rc;

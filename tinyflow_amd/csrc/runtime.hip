@@ -316,6 +316,7 @@ extern "C" int DLArrayAlloc(const index_t *shape, index_t ndim_in, DLContext ctx
   size_t bytes = sizeof(float);
   for (int i = 0; i < ndim; ++i) {
     TF_REQUIRE(shape[i] >= 0, "negative extent");
+    TF_REQUIRE(shape[i] == 0 || bytes <= ((size_t)1 << 62) / (size_t)shape[i], "shape overflows the address space");
     bytes *= (size_t)shape[i];
   }
   void *data = nullptr;
@@ -327,7 +328,7 @@ extern "C" int DLArrayAlloc(const index_t *shape, index_t ndim_in, DLContext ctx
   }
   if (!data) {
     // out-of-memory convention of the reference: report the size, leave *out alone
-    if (memorytoSaving) *memorytoSaving = (int)bytes;
+    if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
   DLArray *arr = new DLArray();
