@@ -347,6 +347,14 @@ int DLGpuAdam_mv(DLArrayHandle m, DLArrayHandle v, const DLArrayHandle g,
 int DLGpuAdam(DLArrayHandle output, const DLArrayHandle m, const DLArrayHandle v,
               float b1t, float b2t, float e, float learning_rate, void **stream);
 
+/* Fused multi-tensor Adam: one launch and one pass over (w, m, v, g) of every
+ * parameter tensor, addressed through the same index tables as DLGpuSgd_o.
+ * ref: c_runtime_api.h:524-532, 560, gpu_op.cu:4674-4700, 4745-4781, 4865-4893 */
+int DLGpuGetN4CudaPointer(void **output, void **m, void **v, void **g, int number, void ****result);
+int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int count,
+                const float b1, const float b2, const float b1t, const float b2t,
+                const float e, const float learning_rate);
+
 #ifdef __cplusplus
 }
 #endif

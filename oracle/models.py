@@ -211,3 +211,23 @@ def train_step(net, params, X, y_onehot, lr):
     net.backward(O.softmax_cross_entropy_gradient(logits, y_onehot, 1.0), grads, need_dx=False)
     new_params = {k: O.sgd_update(v, grads[k], lr) for k, v in params.items()}
     return loss, grads, new_params, logits
+
+
+def train_step_adam(net, params, moments, X, y_onehot, lr, step, b1=0.9, b2=0.999, e=1e-8):
+    """One forward + backward + Adam step; ``step`` counts from 1.
+
+    ``moments`` maps a parameter name to (m, v).  Returns (loss, grads, new_params,
+    new_moments).  m, v update: reference gpu_op.cu:4495-4506; parameter update with
+    the bias corrections 1 - b1**step, 1 - b2**step: reference gpu_op.cu:4461-4467 and
+    TrainExecuteAdam.py:16-21, 196-198 (the powers start at b1, b2 and are multiplied
+    once after every step)."""
+    logits = net.forward(X, params)
+    loss = O.softmax_cross_entropy(logits, y_onehot)
+    grads = {}
+    net.backward(O.softmax_cross_entropy_gradient(logits, y_onehot, 1.0), grads, need_dx=False)
+    new_params, new_moments = {}, {}
+    for k, w in params.items():
+        m, v = O.adam_mv(moments[k][0], moments[k][1], grads[k], b1, b2)
+        new_moments[k] = (m, v)
+        new_params[k] = O.adam_update(w, m, v, b1 ** step, b2 ** step, e, lr)
+    return loss, grads, new_params, new_moments

@@ -252,3 +252,72 @@ def test_add_relu_equals_add_then_relu(rt, shape):
     gpu_op.matrix_elementwise_add_relu(ga, gb, got, rt.stream)
     assert got.asnumpy().tobytes() == want.asnumpy().tobytes()
     assert got.asnumpy().tobytes() == O.relu(O.add(a, b)).tobytes()
+
+
+def test_adam_two_kernel_form(rt):
+    """DLGpuAdam_mv then DLGpuAdam against the written-out formulas (gpu_op.cu:4461-4506)."""
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(31)
+    shape = (257, 33)
+    w, g = rng.normal(0, 1, shape).astype(np.float32), rng.normal(0, 0.1, shape).astype(np.float32)
+    m, v = rng.normal(0, 0.1, shape).astype(np.float32), rng.uniform(0, 0.01, shape).astype(np.float32)
+    gw, gg, gm, gv = (_gpu(a, rt) for a in (w, g, m, v))
+    # the coefficients reach the kernels as C floats: the oracle gets the same rounded values
+    b1, b2, b1t, b2t = (float(np.float32(c)) for c in (0.9, 0.999, 0.9 ** 3, 0.999 ** 3))
+    gpu_op.adam_mv(gm, gv, gg, b1, b2, rt.stream)
+    m_ref, v_ref = O.adam_mv(m.astype(np.float64), v.astype(np.float64), g.astype(np.float64), b1, b2)
+    np.testing.assert_allclose(gm.asnumpy(), m_ref, rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(gv.asnumpy(), v_ref, rtol=1e-6, atol=1e-10)
+    gpu_op.adam_compute(gw, gm, gv, b1t, b2t, 1e-8, 0.001, rt.stream)
+    w_ref = O.adam_update(w.astype(np.float64), m_ref, v_ref, b1t, b2t, 1e-8, 0.001)
+    np.testing.assert_allclose(gw.asnumpy(), w_ref, rtol=1e-5, atol=1e-7)
+
+
+def _flat_index_tables(sizes):
+    """index -> (tensor number, offset inside it) for tensors laid end to end, the
+    tables DLGpuSgd_o / DLGpuAdam_o walk (gpu_op.cu:4824-4836)."""
+    number = np.concatenate([np.full(n, t, dtype=np.int32) for t, n in enumerate(sizes)])
+    offset = np.concatenate([np.arange(n, dtype=np.int32) for n in sizes])
+    return [int(i) for i in number], [int(i) for i in offset]
+
+
+def test_fused_multi_tensor_sgd_and_adam(rt):
+    """One launch over all parameter tensors equals the per-tensor entry points bit for
+    bit (same arithmetic per element; Adam: same expressions as the two-kernel form)."""
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(32)
+    shapes = [(64, 3, 3, 3), (10,), (1,), (129, 7), (2, 2)]
+    sizes = [int(np.prod(s)) for s in shapes]
+    number, offset = _flat_index_tables(sizes)
+    count = len(number)
+    tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, count)
+
+    def fresh():
+        r = np.random.RandomState(33)
+        return [[_gpu(r.normal(0, 1, s) if k != 2 else r.uniform(0, 0.01, s), rt) for s in shapes]
+                for k in range(4)]   # w, m, v, g
+
+    def pointers(arrays):
+        return [a.handle.contents.data for a in arrays]
+
+    # SGD
+    w1, _, _, g1 = fresh()
+    w2, _, _, g2 = fresh()
+    for w, g in zip(w1, g1):
+        gpu_op.sgd_update(w, g, 0.05, rt.stream)
+    n2 = gpu_op.get_n2_cuda_pointer(pointers(w2), pointers(g2), len(shapes))
+    gpu_op.sgd_compute_o(n2, tables, count, 0.05)
+    for a, b in zip(w1, w2):
+        np.testing.assert_array_equal(a.asnumpy(), b.asnumpy())
+    # Adam
+    w1, m1, v1, g1 = fresh()
+    w2, m2, v2, g2 = fresh()
+    b1t, b2t = 0.9 ** 2, 0.999 ** 2
+    for w, m, v, g in zip(w1, m1, v1, g1):
+        gpu_op.adam_mv(m, v, g, 0.9, 0.999, rt.stream)
+        gpu_op.adam_compute(w, m, v, b1t, b2t, 1e-8, 0.001, rt.stream)
+    n4 = gpu_op.get_n4_cuda_pointer(pointers(w2), pointers(m2), pointers(v2), pointers(g2), len(shapes))
+    gpu_op.adam_compute_o(n4, tables, count, 0.9, 0.999, b1t, b2t, 1e-8, 0.001)
+    for name, one, two in (("m", m1, m2), ("v", v1, v2), ("w", w1, w2)):
+        for a, b in zip(one, two):
+            np.testing.assert_allclose(a.asnumpy(), b.asnumpy(), rtol=2e-7, atol=1e-7, err_msg=name)

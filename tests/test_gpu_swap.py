@@ -216,3 +216,38 @@ def test_planner_lists_drive_the_step_bit_identically():
             assert a.tobytes() == b.tobytes()
     ex.close()
     ex2.close()
+
+
+def test_planner_message_carries_measured_runtimes():
+    """The executor -> planner report after a measured step: every computed node has a
+    positive runtime, the convolutions' runtimes dominate, sizes match the arrays, and
+    the measuring step itself still gives the plain executor's bits."""
+    from tinyflow_amd.SwapExecute import SwapExecutor
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    model, X, y = _shallow_resnet()
+    plain = TrainExecutor(model.loss, 0.01)
+    plain.init_Variable(dict(model.variables))
+    want = [o.asnumpy() for o in plain.run({model.X: X, model.y_: y})]
+
+    model, X, y = _shallow_resnet()
+    ex = SwapExecutor(model.loss, 0.01, swap=False)
+    ex.init_Variable(dict(model.variables))
+    ex.measure_runtimes = True
+    got = [o.asnumpy() for o in ex.run({model.X: X, model.y_: y})]
+    ex.measure_runtimes = False
+    for a, b in zip(want, got):
+        assert a.tobytes() == b.tobytes()
+    msg = ex.planner_message()
+    assert len(msg) == len(ex.topo_order)
+    by_kind = {}
+    for node, (tensors, inputs, name, op_id, flag, _, runtime) in zip(ex.topo_order, msg):
+        if node.isw in (1, 2):
+            assert runtime == 1e-8            # fed, not computed
+            continue
+        assert 1e-8 <= runtime < 0.5, (name, runtime)
+        by_kind[type(node.op).__name__] = by_kind.get(type(node.op).__name__, 0.0) + runtime
+        if not node.issgd:
+            assert tensors[0][1] == 4 * int(np.prod(ex.tensors[node].shape))
+    conv = sum(v for k, v in by_kind.items() if k.startswith("Convolution"))
+    assert conv > 0 and conv >= 0.2 * sum(by_kind.values()), by_kind
+    ex.close()

@@ -161,3 +161,57 @@ def test_fused_bn_relu_executor_is_bit_identical():
     for a_step, b_step in zip(*runs):
         for a, b in zip(a_step, b_step):
             assert a.tobytes() == b.tobytes()
+
+
+@pytest.mark.parametrize("config", ["mlp", "lenet5"])
+def test_adam_executor_matches_oracle(config):
+    """Three Adam steps (the reference's TrainExecuteAdam flow): loss, gradients, both
+    moments and the parameters against the float64 oracle.
+
+    MLP: elementwise rtol 1e-3.  The update divides by sqrt(v) + 1e-8, so a gradient
+    entry of magnitude below ~1e-6 turns its own rounding error into an update error of
+    up to lr; parameters therefore get an absolute bound of lr * 1e-2 on top of rtol.
+    LeNet-5: Adam moves every weight by about +-lr per step whatever its gradient, which
+    now and then leaves two candidates of a max-pool window within rounding of each
+    other; float32 and float64 then route one dy differently and the conv gradients
+    move by ~5e-3 in relative L2 (the float32 evaluation of the oracle shows the same
+    against float64 at step 3 of this very case).  Tensors are therefore compared in
+    relative L2 with a bound of 2e-2; a wiring error is O(1)."""
+    from tinyflow_amd import models
+    from tinyflow_amd.TrainExecuteAdam import TrainExecutor
+    lr = 0.001
+    model, X, y = models.build(config)
+    ex = TrainExecutor(model.loss, lr)
+    ex.init_Variable(dict(model.variables))
+    names = [v.name for v in model.variables]
+    by_name = {v.name: v for v in model.variables}
+    params = {v.name: val.astype(np.float64) for v, val in model.variables.items()}
+    moments = {k: (np.zeros_like(w), np.zeros_like(w)) for k, w in params.items()}
+    net = OM.network(config)
+    grad_nodes = dict(zip(ex.Variable_node_list, ex.Variable_node_grad_list))
+    X64, y64 = X.astype(np.float64), y.astype(np.float64)
+    elementwise = config == "mlp"
+    for step in range(1, 4):
+        out = ex.run({model.X: X, model.y_: y})
+        assert abs(ex.b1t[0] - 0.9 ** (step + 1)) < 1e-12 and abs(ex.b2t[0] - 0.999 ** (step + 1)) < 1e-12
+        loss_ref, grads_ref, params, moments = OM.train_step_adam(net, params, moments, X64, y64, lr, step)
+        _close(out[0].asnumpy(), loss_ref, "%s step %d loss" % (config, step), rtol=1e-4)
+        for name, arr in zip(names, out[1:1 + len(names)]):
+            what = "%s step %d %s" % (config, step, name)
+            grad = ex.value_of(grad_nodes[by_name[name]]).asnumpy()
+            m, v = (a.asnumpy() for a in ex.moments_of(by_name[name]))
+            if elementwise:
+                _close(grad, grads_ref[name], what + " grad")
+                _close(m, moments[name][0], what + " m")
+                _close(v, moments[name][1], what + " v", atol=1e-9)
+                np.testing.assert_allclose(arr.asnumpy().astype(np.float64), params[name], rtol=1e-3,
+                                           atol=lr * 1e-2, err_msg=what + " param")
+            else:
+                for got, ref, part, bound in ((grad, grads_ref[name], "grad", 2e-2), (m, moments[name][0], "m", 2e-2),
+                                              (v, moments[name][1], "v", 4e-2), (arr.asnumpy(), params[name], "param", 1e-3)):
+                    err = _rel_err(got, ref)
+                    assert err <= bound, "%s %s: relative L2 error %.3g > %.3g" % (what, part, err, bound)
+        # continue from the GPU's own state so that the next step compares like with like
+        params = {name: arr.asnumpy().astype(np.float64) for name, arr in zip(names, out[1:1 + len(names)])}
+        moments = {name: tuple(a.asnumpy().astype(np.float64) for a in ex.moments_of(by_name[name]))
+                   for name in names}

@@ -247,6 +247,30 @@ def test_updates_are_placed_behind_the_last_reader(config, kw):
         assert all(pos[i] < pos[n] for i in n.inputs)
 
 
+def test_adam_updates_are_placed_behind_the_last_reader():
+    """The Adam step graph: one update node per variable reading (w, m, v, grad), two
+    zero-initialised moment variables per variable, updates behind the last reader."""
+    from tinyflow_amd import TrainExecuteAdam as A
+    model, _, _ = models.build("lenet5")
+    var_list = list(reversed(ad.get_Variable_node_list(model.loss)))
+    b1t, b2t = [0.9], [0.999]
+    updates, mv, var_to_mv = A.getcomputelist(var_list, ad.gradients(model.loss, var_list), 0.9, 0.999, b1t, b2t,
+                                              1e-8, 0.001)
+    assert len(updates) == len(var_list) and len(mv) == 2 * len(var_list)
+    for upd, var in zip(updates, var_list):
+        m, v = var_to_mv[var]
+        assert upd.inputs[:3] == [var, m, v] and upd.issgd == 1
+        assert (m.name, v.name, m.isw, v.isw) == (var.name + "m", var.name + "v", 1, 1)
+        assert upd.b1t is b1t and upd.b2t is b2t          # shared with the executor, which advances them
+    order = A.swapadam(ad.find_topo_sort(updates))
+    pos = {n: i for i, n in enumerate(order)}
+    for upd in updates:
+        readers = [n for n in order if not n.issgd and upd.inputs[0] in n.inputs]
+        assert readers and max(pos[r] for r in readers) < pos[upd]
+    for n in order:
+        assert all(pos[i] < pos[n] for i in n.inputs)
+
+
 def test_resnet50_graph_census():
     """ResNet-50 as the reference builds it: 53 convolutions and 53 batch norms, 49
     ReLUs, 16 residual adds; the first convolution's grad-data node is never reached
@@ -345,6 +369,48 @@ def test_planner_wire_format_round_trip():
     assert releases == [(4, 0), (25, 1), (25, 2), (25, 5)]
     out2, in2, rel2, rec2 = schedule_from_wire(swaps, releases, [(9, 4, True)])
     assert out2 == swap_out and in2 == swap_in and rel2 == release and rec2 == {9: [4]}
+
+
+def test_planner_message_format():
+    """Executor -> planner report (reference autodiff.py:2473-2510): one entry per node,
+    ids are topological positions, update nodes list the tensors they rewrite under
+    id + node count, parameters and the loss carry the flag."""
+    from tinyflow_amd import TrainExecuteAdam as A
+    from tinyflow_amd.SwapExecute import planner_message
+    from tinyflow_amd.TrainExecute import getcomputelist, swapsgd
+    model, X, y = models.build("lenet5")
+    variables = list(reversed(ad.get_Variable_node_list(model.loss)))
+    grads = ad.gradients(model.loss, variables)
+    for optimizer in ("sgd", "adam"):
+        if optimizer == "sgd":
+            updates = getcomputelist(variables, grads, 0.1)
+            fed = {}
+        else:
+            updates, mv, var_to_mv = A.getcomputelist(variables, grads, 0.9, 0.999, [0.9], [0.999], 1e-8, 0.001)
+            fed = {n: np.shape(model.variables[v]) for v, pair in var_to_mv.items() for n in pair}
+        topo = swapsgd(ad.find_topo_sort(updates))
+        shapes = {model.X: X.shape, model.y_: y.shape}
+        shapes.update({v: np.shape(val) for v, val in model.variables.items()})
+        shapes.update(fed)
+        for n in topo:
+            if n not in shapes:
+                shapes[n] = tuple(n.op.infer_shape(n, [shapes[i] for i in n.inputs], None))
+        some = topo[len(topo) // 2]
+        msg = planner_message(topo, shapes, model.loss, {some: 2.5e-4})
+        assert len(msg) == len(topo)
+        total = len(topo)
+        for i, (node, entry) in enumerate(zip(topo, msg)):
+            tensors, inputs, name, op_id, flag, empty, runtime = entry
+            assert (name, op_id, empty) == (node.name, i, [])
+            assert inputs == [topo.index(p) for p in node.inputs]
+            assert flag == (1 if (node.isw == 1 or node is model.loss) else 0)
+            assert runtime == (2.5e-4 if node is some else 1e-8)
+            if node.issgd:
+                want = 3 if optimizer == "adam" else 1
+                assert [t[0] for t in tensors] == [topo.index(p) + total for p in node.inputs[:want]]
+                assert all(t[1] == 4 * int(np.prod(shapes[p])) for t, p in zip(tensors, node.inputs))
+            else:
+                assert tensors == [(i, 4 * int(np.prod(shapes[node])), tuple(shapes[node]))]
 
 
 def test_recompute_schedule_invariants():

@@ -281,6 +281,32 @@ def schedule_from_wire(swap_list, release_list, recompute_list=()):
     return swap_out, swap_in, release, recompute
 
 
+def planner_message(topo_order, shapes, loss, runtimes=None):
+    """What the executor reports to the planner before it asks for a schedule
+    (pycode/tinyflow/autodiff.py:2473-2510): one entry per node, in topological order,
+    ``[tensor_list, input_ids, op_name, op_id, is_input_or_output, [], runtime]`` with
+    ``tensor_list = [(tensor_id, nbytes, shape)]``.  Ids are positions in the
+    topological order.  An in-place update node owns no tensor of its own: it lists
+    the tensors it rewrites (parameter; for Adam also the two moments) under
+    ``id + len(topo_order)``, as the reference does for its Adam nodes.  The flag is 1
+    for parameters and for the loss.  ``runtimes`` maps a node to seconds; nodes it
+    does not cover get the reference's placeholder of 1e-8 s (1e-5 ms)."""
+    pos = {n: i for i, n in enumerate(topo_order)}
+    total = len(topo_order)
+    runtimes = runtimes or {}
+    message = []
+    for node in topo_order:
+        if node.issgd:
+            rewritten = node.inputs[:3] if isinstance(node.op, ad.AdamOp) else node.inputs[:1]
+            tensors = [(pos[i] + total, 4 * int(np.prod(shapes[i])), tuple(shapes[i])) for i in rewritten]
+        else:
+            tensors = [(pos[node], 4 * int(np.prod(shapes[node])), tuple(shapes[node]))]
+        flag = 1 if (node.isw == 1 or node is loss) else 0
+        message.append([tensors, [pos[i] for i in node.inputs], node.name, pos[node], flag, [],
+                        float(runtimes.get(node, 1e-8))])
+    return message
+
+
 class SwapExecutor(object):
     """SGD step executor that keeps the device footprint small by releasing dead
     values and swapping forward activations to pinned host memory."""
@@ -312,6 +338,34 @@ class SwapExecutor(object):
         self.prefetcher.start()
         self.stats = {}
         self.wire_schedule = None
+        self.measure_runtimes = False   # time every node of the next steps (waits for the device around each)
+        self.node_runtime = {}          # node -> seconds, filled while measure_runtimes is set
+        self._sync_cell = None
+
+    def _device_sync(self):
+        """Wait until everything enqueued so far has run (a synchronous one-element read)."""
+        if self._sync_cell is None:
+            self._sync_cell = ndarray.array(np.zeros(1, np.float32), ctx=self.ctx)
+        self._sync_cell.asnumpy()
+
+    def _idle_sync_seconds(self):
+        """Cost of ``_device_sync`` on an idle device, subtracted from measured runtimes."""
+        self._device_sync()
+        best = 1.0
+        for _ in range(5):
+            started = time.perf_counter()
+            self._device_sync()
+            best = min(best, time.perf_counter() - started)
+        return best
+
+    def planner_message(self, runtimes=None):
+        """The per-node report a planner builds its schedule from (see the module-level
+        ``planner_message``); call after the first step, when shapes are known.  Uses
+        the runtimes measured under ``measure_runtimes`` unless others are given."""
+        assert self.tensors is not None, "run one step first: shapes are inferred there"
+        shapes = {n: t.shape for n, t in self.tensors.items()}
+        return planner_message(self.topo_order, shapes, self.targetloss,
+                               self.node_runtime if runtimes is None else runtimes)
 
     def set_schedule(self, swap_list, release_list, recompute_list=()):
         """Run the steps from a planner's lists (the wire format described at
@@ -442,6 +496,7 @@ class SwapExecutor(object):
             else:
                 t.gpu._sync_copyfrom(value)
         handles = self._handles = (self.cudnnHandle, self.cublasHandle, self.cudaStream)
+        sync_cost = self._idle_sync_seconds() if self.measure_runtimes else 0.0
         for t in self.tensors.values():
             if t.state == HOST and t.node not in self.keep:
                 t.state = FREED   # last step's host copy is stale
@@ -457,7 +512,13 @@ class SwapExecutor(object):
                 out = None
                 if not node.issgd:
                     out = self._alloc(t.shape, node.name, node.inputs)
+                if self.measure_runtimes:
+                    self._device_sync()
+                    started = time.perf_counter()
                 wanted = node.op.compute(node, input_vals, out, *handles)
+                if self.measure_runtimes:
+                    self._device_sync()
+                    self.node_runtime[node] = max(1e-8, time.perf_counter() - started - sync_cost)
                 for _ in range(3):
                     if not wanted:
                         break

@@ -33,8 +33,7 @@ class TrainExecutor(object):
         self.Variable_node_list = ad.get_Variable_node_list(targetloss)
         self.Variable_node_list.reverse()
         self.Variable_node_grad_list = ad.gradients(targetloss, self.Variable_node_list)
-        self.eval_node_list = getcomputelist(self.Variable_node_list, self.Variable_node_grad_list,
-                                             learning_rate)
+        self.eval_node_list = self._update_nodes()
         self.ctx = ctx
         self.topo_order = swapsgd(ad.find_topo_sort(self.eval_node_list))
         self.node_to_shape_map = None
@@ -45,6 +44,10 @@ class TrainExecutor(object):
         self.cublasHandle = gpu_op.create_cublasHandle(self.cudaStream)
         self.isfirstrun = 0
         self._plan = None
+
+    def _update_nodes(self):
+        """One in-place update node per variable, in ``Variable_node_list`` order."""
+        return getcomputelist(self.Variable_node_list, self.Variable_node_grad_list, self.learning_rate)
 
     def infer_shape(self, feed_shapes):
         """Shapes of every node from the shapes of the fed nodes."""

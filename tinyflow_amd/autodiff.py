@@ -838,6 +838,31 @@ class SgdOp(Op):
         return input_shapes[0]
 
 
+class AdamOp(Op):
+    """In-place Adam update of a parameter and its two moment variables; produces no
+    value of its own (reference autodiff.py:2050-2076).  Inputs: parameter, m, v,
+    gradient.  ``b1t`` / ``b2t`` are one-element lists shared with the executor,
+    which multiplies them by b1 / b2 after every step."""
+
+    def __call__(self, node_A, node_B, node_C, node_D, b1, b2, b1t, b2t, e, learning_rate):
+        node = Op.__call__(self)
+        node.inputs = [node_A, node_B, node_C, node_D]
+        node.name = "AdamOp"
+        node.b1, node.b2, node.b1t, node.b2t, node.e = b1, b2, b1t, b2t, e
+        node.learning_rate = learning_rate
+        return node
+
+    def compute(self, node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream, use_numpy=False):
+        _no_numpy(use_numpy)
+        gpu_op.adam_mv(input_vals[1], input_vals[2], input_vals[3], node.b1, node.b2, cudaStream)
+        gpu_op.adam_compute(input_vals[0], input_vals[1], input_vals[2], node.b1t[0], node.b2t[0], node.e,
+                            node.learning_rate, cudaStream)
+        return 0
+
+    def infer_shape(self, node, input_shapes, cudnnHandle):
+        return input_shapes[0]
+
+
 # ------------------------------------------------------------------- composites
 
 def dense(X, W, b):
@@ -1022,6 +1047,7 @@ bn_forward_op = BNForwardOp()
 bn_backward_op = BNBackwardOp()
 fullybn_forward_op = FullyBNForwardOp()
 sgd_op = SgdOp()
+adam_op = AdamOp()
 dropout_forward_op = DropoutForwardOp()
 dropout_backward_op = DropoutBackwardOp()
 fullydropout_forward_op = FullyDropoutForwardOp()

@@ -108,6 +108,26 @@ __global__ __launch_bounds__(kThreads) void sgd_multi_kernel(float **w, float **
   }
 }
 
+// Fused multi-tensor Adam over the same flat index space, one lane per parameter
+// and one pass over w, m, v, g (28 bytes per parameter):
+//   m = b1*m + (1-b1)*g;  v = b2*v + (1-b2)*g*g
+//   w -= (lr * m / (1-b1t)) / (sqrt(v / (1-b2t)) + e)
+__global__ __launch_bounds__(kThreads) void adam_multi_kernel(float **w, float **m, float **v, float **g,
+                                                             const int *__restrict__ number,
+                                                             const int *__restrict__ offset, float b1, float b2,
+                                                             float b1t, float b2t, float e, float lr, int count) {
+  const int stride = gridDim.x * kThreads;
+  for (int i = blockIdx.x * kThreads + threadIdx.x; i < count; i += stride) {
+    const int t = number[i], o = offset[i];
+    const float gi = g[t][o];
+    const float mm = m[t][o] * b1 + gi * (1.f - b1);
+    const float vv = v[t][o] * b2 + gi * gi * (1.f - b2);
+    m[t][o] = mm;
+    v[t][o] = vv;
+    w[t][o] = w[t][o] - (lr * mm / (1.f - b1t)) / (sqrtf(vv / (1.f - b2t)) + e);
+  }
+}
+
 }  // namespace
 
 extern "C" int DLGpuArraySet(DLArrayHandle arr, float value, void **stream) {
@@ -303,6 +323,33 @@ extern "C" int DLGpuGetN2CudaPointer(void **output, void **g, int number, void *
   (*result)[0] = (void **)d_out;
   (*result)[1] = (void **)d_g;
   return 0;
+}
+
+extern "C" int DLGpuGetN4CudaPointer(void **output, void **m, void **v, void **g, int number, void ****result) {
+  TF_REQUIRE(output && m && v && g && result && number >= 0, "bad arguments");
+  void **host[4] = {output, m, v, g};
+  float **dev[4] = {nullptr, nullptr, nullptr, nullptr};
+  const size_t bytes = sizeof(float *) * (size_t)(number > 0 ? number : 1);
+  for (int i = 0; i < 4; ++i) {
+    TF_HIP(hipMalloc((void **)&dev[i], bytes));
+    TF_HIP(hipMemcpy(dev[i], host[i], sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
+  }
+  *result = (void ***)malloc(sizeof(void **) * 4);
+  for (int i = 0; i < 4; ++i) (*result)[i] = (void **)dev[i];
+  return 0;
+}
+
+extern "C" int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int count, const float b1,
+                           const float b2, const float b1t, const float b2t, const float e,
+                           const float learning_rate) {
+  TF_REQUIRE(n4list && *n4list && indexlist && *indexlist && count >= 0, "bad arguments");
+  if (count == 0) return 0;
+  // no stream argument: default stream, ordered against all created streams
+  hipLaunchKernelGGL(adam_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, nullptr,
+                     (float **)((*n4list)[0]), (float **)((*n4list)[1]), (float **)((*n4list)[2]),
+                     (float **)((*n4list)[3]), (const int *)((*indexlist)[0]), (const int *)((*indexlist)[1]), b1,
+                     b2, b1t, b2t, e, learning_rate, count);
+  return finish(nullptr, "DLGpuAdam_o");
 }
 
 extern "C" int DLGpuSgd_o(void ****n2list, const void ***indexlist, const int count,

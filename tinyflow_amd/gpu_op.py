@@ -395,8 +395,22 @@ def get_n2_cuda_pointer(output, g, number):
     return result
 
 
+def get_n4_cuda_pointer(output, m, v, g, number):
+    result = _cell(4)
+    check_call(_LIB.DLGpuGetN4CudaPointer(c_array(ctypes.c_void_p, output), c_array(ctypes.c_void_p, m),
+                                          c_array(ctypes.c_void_p, v), c_array(ctypes.c_void_p, g),
+                                          ctypes.c_int(number), result))
+    return result
+
+
 def sgd_compute_o(n2list, indexinfolist, count, learning_rate):
     check_call(_LIB.DLGpuSgd_o(n2list, indexinfolist, ctypes.c_int(count), ctypes.c_float(learning_rate)))
+
+
+def adam_compute_o(n4list, indexinfolist, count, b1, b2, b1t, b2t, e, learning_rate):
+    check_call(_LIB.DLGpuAdam_o(n4list, indexinfolist, ctypes.c_int(count), ctypes.c_float(b1),
+                                ctypes.c_float(b2), ctypes.c_float(b1t), ctypes.c_float(b2t),
+                                ctypes.c_float(e), ctypes.c_float(learning_rate)))
 
 
 def getInt(intp):
