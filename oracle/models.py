@@ -231,3 +231,25 @@ def train_step_adam(net, params, moments, X, y_onehot, lr, step, b1=0.9, b2=0.99
         new_moments[k] = (m, v)
         new_params[k] = O.adam_update(w, m, v, b1 ** step, b2 ** step, e, lr)
     return loss, grads, new_params, new_moments
+
+
+def train_step_cross_head(net, params, X, y_onehot, lr):
+    """One forward + backward + SGD step with the loss head of the reference's
+    ``*_leo`` model scripts (pycode/tinyflow/VGG16_test_leo.py:250-254) on top of
+    ``net``'s logits: per-feature batch norm over the batch, softmax per instance,
+    loss = sum(-y_ * log(p)) / p.size (reference autodiff.py:2079-2103, 2153-2156),
+    differentiated link by link: cross backward (gpu_op.cu:4568-4573), softmax
+    backward (gpu_op.cu:3521-3531), batch-norm backward, then the network.
+    Returns (loss, grads, new_params)."""
+    logits = net.forward(X, params)
+    z, mean, istd = O.batch_norm_forward(logits, "pre_activation")
+    p = O.activation_forward(z, "softmax")
+    scale = 1.0 / p.size
+    loss = np.sum(O.cross(p, y_onehot, scale)).reshape(1)
+    dp = O.cross_backward(p, y_onehot, np.ones_like(p), scale)
+    dz = O.activation_backward(z, p, dp, "softmax")
+    dlogits = O.batch_norm_backward(logits, dz, "pre_activation", mean, istd)
+    grads = {}
+    net.backward(dlogits, grads, need_dx=False)
+    new_params = {k: O.sgd_update(v, grads[k], lr) for k, v in params.items()}
+    return loss, grads, new_params

@@ -321,3 +321,22 @@ def test_fused_multi_tensor_sgd_and_adam(rt):
     for name, one, two in (("m", m1, m2), ("v", v1, v2), ("w", w1, w2)):
         for a, b in zip(one, two):
             np.testing.assert_allclose(a.asnumpy(), b.asnumpy(), rtol=2e-7, atol=1e-7, err_msg=name)
+
+
+@pytest.mark.parametrize("shape", [(128, 10), (32, 1000), (7, 3)])
+def test_cross_and_its_gradient(rt, shape):
+    """DLGpuCross / DLGpuCrossBackward: -b * y * log(x) and -b * y / x * dout
+    (gpu_op.cu:4538-4597)."""
+    from tinyflow_amd import gpu_op
+    rng = np.random.RandomState(34)
+    x = rng.uniform(0.01, 1.0, shape).astype(np.float32)
+    y = np.zeros(shape, np.float32)
+    y[np.arange(shape[0]), rng.randint(0, shape[1], shape[0])] = 1.0
+    dout = rng.normal(0, 1, shape).astype(np.float32)
+    b = 1.0 / x.size
+    out, dx = _empty(shape, rt), _empty(shape, rt)
+    gpu_op.cross(_gpu(x, rt), _gpu(y, rt), out, b, rt.stream)
+    np.testing.assert_allclose(out.asnumpy(), O.cross(x.astype(np.float64), y, b), rtol=1e-5, atol=1e-12)
+    gpu_op.cross_backward(_gpu(x, rt), _gpu(y, rt), _gpu(dout, rt), dx, b, rt.stream)
+    np.testing.assert_allclose(dx.asnumpy(), O.cross_backward(x.astype(np.float64), y, dout.astype(np.float64), b),
+                               rtol=1e-5, atol=1e-12)

@@ -215,3 +215,43 @@ def test_adam_executor_matches_oracle(config):
         params = {name: arr.asnumpy().astype(np.float64) for name, arr in zip(names, out[1:1 + len(names)])}
         moments = {name: tuple(a.asnumpy().astype(np.float64) for a in ex.moments_of(by_name[name]))
                    for name in names}
+
+
+@pytest.mark.parametrize("config", ["mlp", "lenet5"])
+def test_cross_entropy_loss_head_matches_oracle(config):
+    """The loss head of the reference's model scripts -- batch norm of the logits,
+    softmax activation, cross / reduce-sum -- through the step executor: loss, every
+    gradient and every updated parameter for two steps against the float64 oracle,
+    which differentiates the head link by link.  The oracle's result is also checked
+    against the closed form dz = (p - y_) / p.size for one-hot labels."""
+    from oracle import ops as O
+    from tinyflow_amd import models
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    lr = 0.5   # the head's gradient carries 1 / (N * classes): a large rate keeps the update visible
+    model, X, y = models.build(config, head="cross")
+    ex = TrainExecutor(model.loss, lr)
+    ex.init_Variable(dict(model.variables))
+    names = [v.name for v in model.variables]
+    params = {v.name: val.astype(np.float64) for v, val in model.variables.items()}
+    net = OM.network(config)
+    grad_nodes = dict(zip(ex.Variable_node_list, ex.Variable_node_grad_list))
+    X64, y64 = X.astype(np.float64), y.astype(np.float64)
+    # closed form of the softmax + cross part for one-hot labels
+    z = np.random.RandomState(5).normal(0, 1, y64.shape)
+    p = O.activation_forward(z, "softmax")
+    dz = O.activation_backward(z, p, O.cross_backward(p, y64, np.ones_like(p), 1.0 / p.size), "softmax")
+    np.testing.assert_allclose(dz, (p - y64) / p.size, rtol=1e-10, atol=1e-15)
+    for step in range(2):
+        out = ex.run({model.X: X, model.y_: y})
+        loss_ref, grads_ref, params = OM.train_step_cross_head(net, params, X64, y64, lr)
+        _close(out[0].asnumpy(), loss_ref, "%s step %d loss" % (config, step), rtol=1e-4)
+        # one scale for all tensors: the last bias gradient is zero in exact arithmetic
+        # (the batch norm on the logits removes any per-class shift), and in float32 it
+        # is the rounding residue of a sum of 1/sqrt(var + eps)-amplified terms, about
+        # 1.5e-5 of the largest gradient entry -- hence atol 5e-5 rather than 1e-5
+        scale = max(float(np.abs(g).max()) for g in grads_ref.values())
+        for name, arr in zip(names, out[1:1 + len(names)]):
+            what = "%s step %d %s" % (config, step, name)
+            got = ex.value_of(grad_nodes[[v for v in model.variables if v.name == name][0]]).asnumpy()
+            np.testing.assert_allclose(got / scale, grads_ref[name] / scale, rtol=1e-3, atol=5e-5, err_msg=what + " grad")
+            _close(arr.asnumpy(), params[name], what + " param")

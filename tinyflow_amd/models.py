@@ -82,7 +82,19 @@ def synthetic_batch(rng, input_shape, n_class, distribution):
     return X.astype(np.float32), y
 
 
-def mlp(rng, batch=128):
+def _loss_head(h, y_, head):
+    """``"softmax_xent"``: the fused softmax cross-entropy node (the benchmark
+    configurations).  ``"cross"``: the head of the reference's ``*_leo`` model scripts
+    (pycode/tinyflow/VGG16_test_leo.py:250-254): batch norm of the logits, softmax
+    activation, then ``crossEntropy_loss`` = sum(-y_ * log(p)) / p.size."""
+    if head == "softmax_xent":
+        return ad.softmaxcrossentropy_op(h, y_)
+    assert head == "cross", head
+    p = ad.fullyactivation_forward_op(ad.fullybn_forward_op(h, "NCHW"), "NCHW", "softmax")
+    return ad.crossEntropy_loss(p, y_)
+
+
+def mlp(rng, batch=128, head="softmax_xent"):
     b = _Builder(rng, init=lambda r, shape: r.normal(0.0, 0.01, shape).astype(np.float32))
     X, y_ = ad.Placeholder("X"), ad.Placeholder("y_")
     h = X
@@ -91,11 +103,11 @@ def mlp(rng, batch=128):
         h = b.dense(h, "fc%d" % (i + 1), sizes[i], sizes[i + 1])
         if i < 2:
             h = ad.relu_op(h)
-    loss = ad.softmaxcrossentropy_op(h, y_)
+    loss = _loss_head(h, y_, head)
     return Model("mlp", loss, h, X, y_, b.variables, (batch, 784), 10)
 
 
-def lenet5(rng, batch=64):
+def lenet5(rng, batch=64, head="softmax_xent"):
     b = _Builder(rng)
     X, y_ = ad.Placeholder("X"), ad.Placeholder("y_")
     h = b.conv(X, "conv1", 1, 6, 5, "SAME", 1, bias=True)
@@ -108,7 +120,7 @@ def lenet5(rng, batch=64):
     h = ad.fullyactivation_forward_op(b.dense(h, "fc3", 400, 120), "NCHW", "relu")
     h = ad.fullyactivation_forward_op(b.dense(h, "fc4", 120, 84), "NCHW", "relu")
     h = b.dense(h, "fc5", 84, 10)
-    loss = ad.softmaxcrossentropy_op(h, y_)
+    loss = _loss_head(h, y_, head)
     return Model("lenet5", loss, h, X, y_, b.variables, (batch, 1, 28, 28), 10)
 
 
