@@ -340,3 +340,23 @@ def test_cross_and_its_gradient(rt, shape):
     gpu_op.cross_backward(_gpu(x, rt), _gpu(y, rt), _gpu(dout, rt), dx, b, rt.stream)
     np.testing.assert_allclose(dx.asnumpy(), O.cross_backward(x.astype(np.float64), y, dout.astype(np.float64), b),
                                rtol=1e-5, atol=1e-12)
+
+
+def test_stream_and_handle_life_cycle(rt):
+    """Create / use / destroy a stream with its two handles; a second destroy of the
+    same cell is reported as an error instead of touching freed memory."""
+    from tinyflow_amd import gpu_op
+    stream = gpu_op.create_cudaStream()
+    cudnn, cublas = gpu_op.create_cudnnHandle(stream), gpu_op.create_cublasHandle(stream)
+    a = _gpu(np.arange(6, dtype=np.float32).reshape(2, 3), rt)
+    b = _gpu(np.ones((3, 2), np.float32), rt)
+    c = _empty((2, 2), rt)
+    gpu_op.matrix_multiply(a, False, b, False, c, cublas, stream)
+    np.testing.assert_array_equal(c.asnumpy(), [[3, 3], [12, 12]])
+    gpu_op.destroy_cudnnHandle(cudnn)
+    gpu_op.destroy_cublasHandle(cublas)
+    gpu_op.destroy_cudaStream(stream)
+    with pytest.raises(RuntimeError):
+        gpu_op.destroy_cudnnHandle(cudnn)
+    with pytest.raises(RuntimeError):
+        gpu_op.destroy_cudaStream(stream)
