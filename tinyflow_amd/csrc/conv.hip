@@ -271,6 +271,7 @@ struct StoreScatter {
   int m_extent, n_extent;  // C, N*P*Q
   FastDiv div_pq, div_q;
   int H, W, u, v;
+  bool pairs;  // u = v = 2 with even H and W: every cell is a full, 8-byte aligned 2 x 2 block
   struct State {
     int col_base[4];
     int rows[4], cols[4];
@@ -292,6 +293,11 @@ struct StoreScatter {
   __device__ inline void store(const State &st, int m, int /*n*/, int j, float val) const {
     if (m < m_extent && st.col_base[j] >= 0) {
       float *cell = out + st.col_base[j] + m * H * W;
+      if (pairs) {  // two 8-byte stores instead of four 4-byte ones
+        *reinterpret_cast<float2 *>(cell) = make_float2(val, 0.f);
+        *reinterpret_cast<float2 *>(cell + W) = make_float2(0.f, 0.f);
+        return;
+      }
       for (int dy = 0; dy < st.rows[j]; ++dy)
         for (int dx = 0; dx < st.cols[j]; ++dx) cell[dy * W + dx] = (dy | dx) == 0 ? val : 0.f;
     }
@@ -677,7 +683,9 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
         launch<BM, BN, BK>(al, bl, ep, K, g, s);
       } else {
         StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
-                        d->H, d->W, d->u, d->v};
+                        d->H, d->W, d->u, d->v,
+                        d->u == 2 && d->v == 2 && d->H % 2 == 0 && d->W % 2 == 0 &&
+                            (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0};
         launch<BM, BN, BK>(al, bl, ep, K, g, s);
       }
     });
