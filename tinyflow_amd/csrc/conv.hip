@@ -361,6 +361,7 @@ struct ConvPlan {
   const char *variant;   // short name of the loader / epilogue combination
   const char *a_loader, *b_loader, *epilogue;  // as they appear in the kernel symbol
   int b_mode;            // MODE template argument of the gathered operand, -1 if none
+  bool a_vec, b_vec;     // operand fetched with the 16-byte loaders (shape permitting)
   int bm, bn, splits;
   int M, N, K;
 };
@@ -443,10 +444,14 @@ ConvPlan plan_forward(const ConvDesc *d) {
   const bool padded = d->pad_h || d->pad_w;
   choose_tile_and_splits(p, false, padded, false, true, 4.0 * p.M * p.N);
   p.variant = padded ? "fwd_pad" : "fwd_nopad";
-  p.a_loader = "PlainAcross";
-  p.b_loader = "GatherAlong";
   p.epilogue = "StoreNCHW";
-  p.b_mode = (d->pad_h || d->pad_w) ? 1 : 0;
+  // filter rows of C*R*S floats; a 1x1 / stride-1 / unpadded input is a plain
+  // [image][channel][pixel] block
+  p.a_vec = p.K % 4 == 0;
+  p.b_vec = p.a_vec && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1 && (d->P * d->Q) % 4 == 0;
+  p.a_loader = p.a_vec ? "Across4" : "PlainAcross";
+  p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
+  p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
   return p;
 }
 
@@ -456,16 +461,19 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   p.M = d->C;
   p.K = d->K * RS;
   p.splits = 1;
-  p.a_loader = "PlainAlong";
-  p.b_loader = "GatherAlong";
   p.epilogue = "StoreNCHW";
   p.b_mode = 0;
+  p.a_vec = d->C % 4 == 0;  // the [(k, r, s)][c] filter has rows of C floats
+  p.b_vec = false;
   if (RS == 1) {
     p.N = d->N * d->P * d->Q;
     const bool dense = d->u == 1 && d->v == 1;
     choose_tile_and_splits(p, false, false, !dense, dense, 4.0 * p.M * d->N * d->H * d->W);
     p.variant = dense ? "dgrad_1x1" : "dgrad_1x1_scatter";
     if (!dense) p.epilogue = "StoreScatter";
+    // dy is read compactly, [image][out channel][pixel]
+    p.b_vec = p.a_vec && (d->P * d->Q) % 4 == 0;
+    p.a_vec = p.b_vec;
   } else {
     p.N = d->N * d->H * d->W;
     if (d->u == 1 && d->v == 1) {
@@ -476,8 +484,12 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
       p.bm = p.bn = 64;
       p.variant = "dgrad_strided";
       p.b_mode = 2;
+      p.a_vec = false;
     }
   }
+  p.a_loader = p.a_vec ? "Along4" : "PlainAlong";
+  p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
+  if (p.b_vec) p.b_mode = -1;
   return p;
 }
 
@@ -489,10 +501,14 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   const bool padded = d->pad_h || d->pad_w;
   choose_tile_and_splits(p, true, padded, false, true, 4.0 * p.M * p.N);
   p.variant = padded ? "wgrad_pad" : "wgrad_nopad";
-  p.a_loader = "DyAcross";
-  p.b_loader = "GatherAcross";
   p.epilogue = "StoreRowMajor";
-  p.b_mode = (d->pad_h || d->pad_w) ? 1 : 0;
+  // dy is [image][out channel][pixel]; x is the same kind of block for a 1x1 /
+  // stride-1 / unpadded filter
+  p.a_vec = (d->P * d->Q) % 4 == 0;
+  p.b_vec = p.a_vec && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1;
+  p.a_loader = p.a_vec ? "Across4" : "DyAcross";
+  p.b_loader = p.b_vec ? "Across4" : "GatherAcross";
+  p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
   return p;
 }
 
@@ -510,9 +526,11 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
   TF_REQUIRE(which >= 0 && which <= 2 && name && name_len > 0, "bad arguments");
   const ConvPlan p = which == 0 ? plan_forward(d) : which == 1 ? plan_dgrad(d) : plan_wgrad(d);
   const int bk = stage_depth(p.bm, p.bn);
-  snprintf(name, (size_t)name_len,
-           "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d>, %s<%d, %d, %d>, %s>", p.variant, p.bm, p.bn,
-           p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, p.b_loader, p.bn, bk, p.b_mode, p.epilogue);
+  char b_args[32];
+  if (p.b_mode >= 0) snprintf(b_args, sizeof b_args, "%d, %d, %d", p.bn, bk, p.b_mode);
+  else snprintf(b_args, sizeof b_args, "%d, %d", p.bn, bk);
+  snprintf(name, (size_t)name_len, "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d>, %s<%s>, %s>", p.variant,
+           p.bm, p.bn, p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, p.b_loader, b_args, p.epilogue);
   if (flops)
     *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
   return 0;
@@ -599,21 +617,37 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
     }
   }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
+  const bool aligned = vec4_ok(filter->data, 0) && vec4_ok(input->data, 0);
+  const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
+  const uint32_t w_bytes = (uint32_t)(numel(filter) * 4), x_bytes = (uint32_t)(numel(input) * 4);
+  const int PQ = d->P * d->Q;
   with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
-    PlainAcross<BM, BK> al{(const float *)filter->data, (uint32_t)(numel(filter) * 4), K, M, K};
-    StoreNCHW ep{partial ? partial : (float *)output->data, M, N, FastDiv((uint32_t)(d->P * d->Q)),
-                 d->P * d->Q, numel(output)};
-    auto run = [&](auto mode_c) {
-      constexpr int MODE = decltype(mode_c)::value;
-      GatherAlong<BN, BK, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4), K, N,
-                               FastDiv((uint32_t)(d->R * d->S)), FastDiv((uint32_t)d->S), d->H * d->W,
-                               FastDiv((uint32_t)(d->P * d->Q)), FastDiv((uint32_t)d->Q),
-                               d->C * d->H * d->W, d->H, d->W, d->u, d->v, -d->pad_h, -d->pad_w,
-                               1, d->R, d->S, FastDiv(1), FastDiv(1)};
-      launch<BM, BN, BK>(al, bl, ep, K, g, s);
+    StoreNCHW ep{partial ? partial : (float *)output->data, M, N, FastDiv((uint32_t)PQ), PQ, numel(output)};
+    auto with_b = [&](const auto &al, auto a_is_vec) {
+      if constexpr (decltype(a_is_vec)::value) {  // a vectorised input only comes with a vectorised filter
+        if (b_vec) {
+          Along4<BN, BK> bl{(const float *)input->data, x_bytes, PQ, N, K, FastDiv((uint32_t)PQ), d->C * PQ};
+          launch<BM, BN, BK>(al, bl, ep, K, g, s);
+          return;
+        }
+      }
+      auto run = [&](auto mode_c) {
+        constexpr int MODE = decltype(mode_c)::value;
+        GatherAlong<BN, BK, MODE> bl{(const float *)input->data, x_bytes, K, N,
+                                 FastDiv((uint32_t)(d->R * d->S)), FastDiv((uint32_t)d->S), d->H * d->W,
+                                 FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
+                                 d->C * d->H * d->W, d->H, d->W, d->u, d->v, -d->pad_h, -d->pad_w,
+                                 1, d->R, d->S, FastDiv(1), FastDiv(1)};
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+      };
+      if (padded) run(IC<1>{}); else run(IC<0>{});
     };
-    if (padded) run(IC<1>{}); else run(IC<0>{});
+    if (a_vec)
+      with_b(Across4<BM, BK>{(const float *)filter->data, w_bytes, K, M, K, FastDiv(ONE_SEGMENT), 0},
+             std::true_type{});
+    else
+      with_b(PlainAcross<BM, BK>{(const float *)filter->data, w_bytes, K, M, K}, std::false_type{});
   });
   if (partial) {
     launch_split_sum(partial, (float *)output->data, numel(output), g.splits, s);
@@ -667,6 +701,9 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   float *dst = partial ? partial : (float *)dinput->data;
   const int64_t dx_count = numel(dinput);
 
+  const bool aligned = vec4_ok(wt, 0) && vec4_ok(doutput->data, 0);
+  const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
+  const FastDiv whole(ONE_SEGMENT);
   if (RS == 1) {
     // 1x1 filter (pad 0): compact GEMM over the output pixels + scatter
     const int N = plan.N;
@@ -674,19 +711,27 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
     with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
       constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
-      PlainAlong<BM, BK> al{wt, w_bytes, d->C, M, K};
-      GatherAlong<BN, BK, 0> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv(1), FastDiv(1), PQ,
-                            FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), d->K * PQ, d->P, d->Q,
-                            1, 1, 0, 0, -1, 1, 1, FastDiv(1), FastDiv(1)};
-      if (d->u == 1 && d->v == 1) {
-        StoreNCHW ep{dst, M, N, FastDiv((uint32_t)PQ), PQ, dx_count};
-        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+      auto with_epilogue = [&](const auto &al, const auto &bl) {
+        if (d->u == 1 && d->v == 1) {
+          StoreNCHW ep{dst, M, N, FastDiv((uint32_t)PQ), PQ, dx_count};
+          launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        } else {
+          StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
+                          d->H, d->W, d->u, d->v,
+                          d->u == 2 && d->v == 2 && d->H % 2 == 0 && d->W % 2 == 0 &&
+                              (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0};
+          launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        }
+      };
+      if (a_vec && b_vec) {
+        with_epilogue(Along4<BM, BK>{wt, w_bytes, d->C, M, K, whole, 0},
+                      Along4<BN, BK>{(const float *)doutput->data, dy_bytes, PQ, N, K, FastDiv((uint32_t)PQ),
+                                     d->K * PQ});
       } else {
-        StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
-                        d->H, d->W, d->u, d->v,
-                        d->u == 2 && d->v == 2 && d->H % 2 == 0 && d->W % 2 == 0 &&
-                            (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0};
-        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        with_epilogue(PlainAlong<BM, BK>{wt, w_bytes, d->C, M, K},
+                      GatherAlong<BN, BK, 0>{(const float *)doutput->data, dy_bytes, K, N, FastDiv(1), FastDiv(1),
+                                             PQ, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), d->K * PQ, d->P,
+                                             d->Q, 1, 1, 0, 0, -1, 1, 1, FastDiv(1), FastDiv(1)});
       }
     });
   } else {
@@ -698,12 +743,12 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
       const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
       with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
         constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
-        PlainAlong<BM, BK> al{wt, w_bytes, d->C, M, K};
         GatherAlong<BN, BK, 1> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv((uint32_t)RS),
                               FastDiv((uint32_t)d->S), PQ,
                               FastDiv((uint32_t)HW), FastDiv((uint32_t)d->W), d->K * PQ, d->P, d->Q,
                               1, 1, d->pad_h, d->pad_w, -1, d->R, d->S, FastDiv(1), FastDiv(1)};
-        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        if (a_vec) launch<BM, BN, BK>(Along4<BM, BK>{wt, w_bytes, d->C, M, K, whole, 0}, bl, ep, K, g, s);
+        else launch<BM, BN, BK>(PlainAlong<BM, BK>{wt, w_bytes, d->C, M, K}, bl, ep, K, g, s);
       });
     } else {
       // strided filter larger than 1x1: every input pixel, taps filtered by divisibility
@@ -754,21 +799,37 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
     dst = partial;
   }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
+  const bool aligned = vec4_ok(doutput->data, 0) && vec4_ok(input->data, 0);
+  const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
+  const uint32_t dy_bytes = (uint32_t)(numel(doutput) * 4), x_bytes = (uint32_t)(numel(input) * 4);
   with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     if constexpr (BM == BN) {  // only the square tiles are used for grad-filter
-      DyAcross<BM, BK> al{(const float *)doutput->data, (uint32_t)(numel(doutput) * 4), K, M,
-                      FastDiv((uint32_t)PQ), d->K * PQ, PQ};
       StoreRowMajor ep{dst, N, M, N, (int64_t)M * N};
-      auto run = [&](auto mode_c) {
-        constexpr int MODE = decltype(mode_c)::value;
-        GatherAcross<BN, BK, MODE> bl{(const float *)input->data, (uint32_t)(numel(input) * 4), K, N,
-                                  FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), FastDiv((uint32_t)RS),
-                                  FastDiv((uint32_t)d->S), d->C * d->H * d->W, d->H * d->W,
-                                  d->H, d->W, d->u, d->v, d->pad_h, d->pad_w};
-        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+      auto with_b = [&](const auto &al, auto a_is_vec) {
+        if constexpr (decltype(a_is_vec)::value) {
+          if (b_vec) {
+            Across4<BN, BK> bl{(const float *)input->data, x_bytes, PQ, N, K, FastDiv((uint32_t)PQ), d->C * PQ};
+            launch<BM, BN, BK>(al, bl, ep, K, g, s);
+            return;
+          }
+        }
+        auto run = [&](auto mode_c) {
+          constexpr int MODE = decltype(mode_c)::value;
+          GatherAcross<BN, BK, MODE> bl{(const float *)input->data, x_bytes, K, N,
+                                    FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q), FastDiv((uint32_t)RS),
+                                    FastDiv((uint32_t)d->S), d->C * d->H * d->W, d->H * d->W,
+                                    d->H, d->W, d->u, d->v, d->pad_h, d->pad_w};
+          launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        };
+        if (padded) run(IC<1>{}); else run(IC<0>{});
       };
-      if (padded) run(IC<1>{}); else run(IC<0>{});
+      if (a_vec)
+        with_b(Across4<BM, BK>{(const float *)doutput->data, dy_bytes, PQ, M, K, FastDiv((uint32_t)PQ), d->K * PQ},
+               std::true_type{});
+      else
+        with_b(DyAcross<BM, BK>{(const float *)doutput->data, dy_bytes, K, M, FastDiv((uint32_t)PQ), d->K * PQ, PQ},
+               std::false_type{});
     }
   });
   if (partial) {

@@ -163,6 +163,124 @@ struct PlainAcross {
   }
 };
 
+// ---- 16-byte loaders ---------------------------------------------------------------
+// One buffer_load_dwordx4 per lane fetches four consecutive elements: a quarter of
+// the load instructions and of the address arithmetic of the one-element loaders
+// above.  Addressing is segmented so that the same two loaders serve plain
+// matrices and the NCHW tensors of 1x1 / stride-1 convolutions (pixels of one image
+// and channel are contiguous, images are `outer` elements apart):
+//   Along4 :  element(d, k) = base[(d / inner) * outer + d % inner + k * ld]
+//   Across4:  element(d, k) = base[d * ld + (k / inner) * outer + k % inner]
+// A plain matrix is the case inner = 2^31 (one segment), outer = 0.
+// Preconditions, checked by the callers: base 16-byte aligned; ld, inner and outer
+// multiples of 4; the extent along the vectorised direction (d for Along4, k for
+// Across4) a multiple of 4, so that a vector is entirely inside or outside.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+constexpr uint32_t ONE_SEGMENT = 0x80000000u;
+__device__ inline f32x4v buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  return __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+}
+inline bool vec4_ok(const void *base, int64_t a, int64_t b = 0, int64_t c = 0, int64_t d = 0) {
+  return (reinterpret_cast<uintptr_t>(base) & 15u) == 0 && a % 4 == 0 && b % 4 == 0 && c % 4 == 0 && d % 4 == 0;
+}
+
+template <int D, int BK>
+struct Along4 {
+  static constexpr int LPR = D / 4;             // lanes per k row of the tile
+  static constexpr int KSTEP = THREADS / LPR;   // k rows covered per pass
+  static constexpr int VPT = BK / KSTEP;        // vector loads per lane per stage
+  static constexpr int EPT = VPT * 4;
+  static_assert(VPT >= 1 && VPT * KSTEP == BK, "tile shape");
+  const float *base;
+  uint32_t bytes;
+  int ld, d_extent, k_extent;
+  FastDiv div_inner;
+  int outer;
+
+  struct State {
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t d_off;  // byte offset of this lane's first d, or OOB
+    int d_local, k_first;
+  };
+  __device__ inline void init(State &st, int origin, int tid) const {
+    st.rsrc = make_rsrc(base, bytes);
+    st.d_local = (tid % LPR) * 4;
+    st.k_first = tid / LPR;
+    const int d = origin + st.d_local;
+    uint32_t seg, rem;
+    div_inner.divmod((uint32_t)(d < d_extent ? d : 0), seg, rem);
+    st.d_off = d < d_extent ? (seg * (uint32_t)outer + rem) * 4u : OOB;
+  }
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
+#pragma unroll
+    for (int e = 0; e < VPT; ++e) {
+      const int k = k0 + st.k_first + e * KSTEP;
+      const uint32_t off = k < k_limit ? st.d_off + (uint32_t)k * (uint32_t)ld * 4u : OOB;
+      const f32x4v v = buf_load4(st.rsrc, off | (st.d_off & OOB));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) reg[4 * e + i] = v[i];
+    }
+  }
+  template <int LD>
+  __device__ inline void store(const State &st, float (*tile)[LD], const float (&reg)[EPT]) const {
+    static_assert(LD % 4 == 0, "rows of the LDS plane must keep 16-byte alignment");
+#pragma unroll
+    for (int e = 0; e < VPT; ++e) {
+      const f32x4v v = {reg[4 * e], reg[4 * e + 1], reg[4 * e + 2], reg[4 * e + 3]};
+      *reinterpret_cast<f32x4v *>(&tile[st.k_first + e * KSTEP][st.d_local]) = v;
+    }
+  }
+};
+
+template <int D, int BK>
+struct Across4 {
+  static constexpr int LPR = BK / 4;            // lanes per d row of the tile
+  static constexpr int DSTEP = THREADS / LPR;
+  static constexpr int VPT = D / DSTEP;
+  static constexpr int EPT = VPT * 4;
+  static_assert(VPT >= 1 && VPT * DSTEP == D, "tile shape");
+  const float *base;
+  uint32_t bytes;
+  int ld, d_extent, k_extent;
+  FastDiv div_inner;
+  int outer;
+
+  struct State {
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t row_off[VPT];  // byte offset of row d, or OOB
+    int k_local, d_first;
+  };
+  __device__ inline void init(State &st, int origin, int tid) const {
+    st.rsrc = make_rsrc(base, bytes);
+    st.k_local = (tid % LPR) * 4;
+    st.d_first = tid / LPR;
+#pragma unroll
+    for (int e = 0; e < VPT; ++e) {
+      const int d = origin + st.d_first + e * DSTEP;
+      st.row_off[e] = d < d_extent ? (uint32_t)d * (uint32_t)ld * 4u : OOB;
+    }
+  }
+  __device__ inline void load(const State &st, int k0, int k_limit, float (&reg)[EPT]) const {
+    const int k = k0 + st.k_local;
+    uint32_t seg, rem;
+    div_inner.divmod((uint32_t)(k < k_limit ? k : 0), seg, rem);
+    const uint32_t k_off = k < k_limit ? (seg * (uint32_t)outer + rem) * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < VPT; ++e) {
+      const f32x4v v = buf_load4(st.rsrc, (st.row_off[e] + k_off) | ((st.row_off[e] | k_off) & OOB));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) reg[4 * e + i] = v[i];
+    }
+  }
+  template <int LD>
+  __device__ inline void store(const State &st, float (*tile)[LD], const float (&reg)[EPT]) const {
+#pragma unroll
+    for (int e = 0; e < VPT; ++e)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tile[st.k_local + i][st.d_first + e * DSTEP] = reg[4 * e + i];
+  }
+};
+
 // ---- epilogue: plain row-major store ---------------------------------------------
 struct StoreRowMajor {
   float *out;

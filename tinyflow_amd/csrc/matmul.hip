@@ -77,6 +77,30 @@ void launch(const AL &al, const BL &bl, const StoreRowMajor &ep, int K, const Ge
 template <int BM, int BN, int BK>
 void dispatch(const float *A, bool tA, int lda, uint32_t a_bytes, const float *B, bool tB, int ldb,
               uint32_t b_bytes, const StoreRowMajor &ep, int M, int N, int K, const Geometry &g, hipStream_t s) {
+  // 16-byte loads when both operands allow them (alignment, leading dimension and
+  // the extent along each operand's contiguous direction multiples of 4)
+  const bool vec = vec4_ok(A, lda, tA ? M : K) && vec4_ok(B, ldb, tB ? K : N);
+  const FastDiv whole(ONE_SEGMENT);
+  if (vec) {
+    if (!tA && !tB) {
+      Across4<BM, BK> al{A, a_bytes, lda, M, K, whole, 0};
+      Along4<BN, BK> bl{B, b_bytes, ldb, N, K, whole, 0};
+      launch<BM, BN, BK>(al, bl, ep, K, g, s);
+    } else if (tA && !tB) {
+      Along4<BM, BK> al{A, a_bytes, lda, M, K, whole, 0};
+      Along4<BN, BK> bl{B, b_bytes, ldb, N, K, whole, 0};
+      launch<BM, BN, BK>(al, bl, ep, K, g, s);
+    } else if (!tA && tB) {
+      Across4<BM, BK> al{A, a_bytes, lda, M, K, whole, 0};
+      Across4<BN, BK> bl{B, b_bytes, ldb, N, K, whole, 0};
+      launch<BM, BN, BK>(al, bl, ep, K, g, s);
+    } else {
+      Along4<BM, BK> al{A, a_bytes, lda, M, K, whole, 0};
+      Across4<BN, BK> bl{B, b_bytes, ldb, N, K, whole, 0};
+      launch<BM, BN, BK>(al, bl, ep, K, g, s);
+    }
+    return;
+  }
   if (!tA && !tB) {
     PlainAcross<BM, BK> al{A, a_bytes, lda, M, K};
     PlainAlong<BN, BK> bl{B, b_bytes, ldb, N, K};
