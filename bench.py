@@ -74,21 +74,23 @@ def stream_handle(stream_cell):
 # commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
 # --config resnet50 --batch 64 only and are reported as null otherwise.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 917379966,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 812899912,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 424364956,
-    "gemm_kernel<128, 128, 16, PlainAlong<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 634931576,
-    "gemm_kernel<128, 128, 16, PlainAcross<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 633969815,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 618614572,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 1153202304,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 516559950,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 340282125,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 840789188,
-    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 474898113,
-    "gemm_kernel<64, 64, 32, PlainAcross<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 337306987,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 346140388,
-    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 505250803,
-    "gemm_kernel<64, 64, 32, DyAcross<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 282734170,
+    "gemm_kernel<128, 128, 16, Along4<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 93080650,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 92895328,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 107179193,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 236793203,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 160938768,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126168592,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 287771063,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89040011,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171063904,
+    "gemm_kernel<64, 128, 16, Along4<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 104529520,
+    "gemm_kernel<64, 128, 16, Across4<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 104363591,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148334962,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 1>, StoreRowMajor>": 90947936,
+    "gemm_kernel<64, 128, 16, PlainAcross<64, 16>, GatherAlong<128, 16, 1>, StoreNCHW>": 244477332,
+    "gemm_kernel<64, 128, 16, Across4<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 79205077,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 112764545,
+    "gemm_kernel<64, 128, 16, PlainAlong<64, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 71179440,
 }
 
 
@@ -287,6 +289,8 @@ def main():
                     help="run the timed steps with batch norm + ReLU evaluated as one kernel each way (an executor "
                          "option outside the reference's op-by-op protocol; bit-identical results).  Without the "
                          "flag the figure is still measured, on a second executor, and reported beside `value`")
+    ap.add_argument("--no-fused-leg", action="store_true",
+                    help="skip the extra measurement of the step with fused batch norm + ReLU (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--no-kernel-events", action="store_true",
@@ -381,8 +385,8 @@ def main():
 
     # The same step with every batch norm + ReLU pair fused, on an executor of its own.
     fused = None
-    if (not args.fuse_bn_relu and not args.mem_limit_gb and args.config.startswith("resnet")
-            and args.bn_mode == "pre_activation"):
+    if (not args.fuse_bn_relu and not args.no_fused_leg and not args.mem_limit_gb
+            and args.config.startswith("resnet") and args.bn_mode == "pre_activation"):
         model2, X2, y2 = models.build(args.config, **kw)
         ex2 = TrainExecutor(model2.loss, 0.01, fuse_bn_relu=True)
         ex2.init_Variable(dict(model2.variables))
