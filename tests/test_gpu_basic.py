@@ -138,6 +138,14 @@ MM_CASES = [
     ((1, 1), False, (1, 1), False),
     ((65, 17), False, (17, 129), False),
     ((33, 130), True, (33, 70), False),
+    # extents that are multiples of 4 but not of a tile (16-byte loaders, all four
+    # transpose cases), and a reduction that is not (one-element loaders)
+    ((132, 36), False, (36, 68), False),
+    ((36, 132), True, (36, 68), False),
+    ((132, 36), False, (68, 36), True),
+    ((36, 132), True, (68, 36), True),
+    ((132, 34), False, (34, 68), False),
+    ((260, 520), False, (520, 388), False),
     # skinny with a long reduction (split-k path)
     ((32, 4096), False, (4096, 1000), False),
     ((64, 2048), False, (2048, 1000), False),

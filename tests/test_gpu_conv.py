@@ -40,6 +40,15 @@ CONV_CASES = [
     (1, 1, 1, 1, 1, 1, 1, "VALID", 1, 1),
     (2, 3, 9, 9, 4, 1, 1, "VALID", 2, 2),        # 1x1 s2 on an odd extent
     (2, 130, 6, 6, 67, 1, 1, "VALID", 3, 3),
+    # around the conditions of the 16-byte loaders (channels, pixels per image multiples of 4 or not)
+    (3, 8, 6, 6, 10, 1, 1, "VALID", 1, 1),       # 1x1, 36 pixels, 8 channels: both operands vectorised
+    (2, 12, 10, 10, 7, 1, 1, "VALID", 1, 1),
+    (2, 6, 8, 8, 10, 1, 1, "VALID", 1, 1),       # 6 channels: one-element loaders
+    (2, 8, 5, 5, 12, 1, 1, "VALID", 1, 1),       # 25 pixels per image: one-element loaders
+    (2, 8, 9, 9, 12, 3, 3, "SAME", 1, 1),        # 3x3: vectorised filter, gathered input, 81 pixels
+    (2, 8, 10, 10, 12, 3, 3, "SAME", 1, 1),      # 100 pixels: vectorised dy in grad-filter
+    (2, 8, 12, 12, 16, 1, 1, "VALID", 2, 2),     # 1x1 s2, even extents: paired scatter stores
+    (130, 4, 2, 2, 4, 1, 1, "VALID", 1, 1),      # many tiny images: a 4-vector per image
 ]
 
 
