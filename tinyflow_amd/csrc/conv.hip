@@ -237,7 +237,8 @@ struct DyAcross {
 };
 
 // ---- epilogues ----------------------------------------------------------------------
-// D[m = channel][n = (img, pixel)] -> out[img][m][pixel]
+// D[m = channel][n = (img, pixel)] -> out[img][m][pixel], through a buffer
+// descriptor (see StoreRowMajor): invalid rows / columns get an out-of-range offset.
 struct StoreNCHW {
   float *out;
   int m_extent, n_extent;
@@ -245,22 +246,23 @@ struct StoreNCHW {
   int HW;
   int64_t split_stride;  // elements between the partial outputs of consecutive k-splits
   struct State {
-    float *base;
-    int col_base[4];  // img * CH * HW + pixel, or -1
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t col_off[4];  // byte offset of (img, channel 0, pixel), or OOB
   };
   template <int TN>
   __device__ inline void init(State &st, int n_wave, int lane, int split) const {
-    st.base = out + (int64_t)split * split_stride;
+    st.rsrc = make_rsrc(out + (int64_t)split * split_stride, (uint32_t)split_stride * 4u);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n_wave + 32 * j + (lane & 31);
       uint32_t img, pix;
       div_hw.divmod((uint32_t)(n < n_extent ? n : 0), img, pix);
-      st.col_base[j] = n < n_extent ? (int)img * m_extent * HW + (int)pix : -1;
+      st.col_off[j] = n < n_extent ? (img * (uint32_t)m_extent * (uint32_t)HW + pix) * 4u : OOB;
     }
   }
   __device__ inline void store(const State &st, int m, int /*n*/, int j, float v) const {
-    if (m < m_extent && st.col_base[j] >= 0) st.base[st.col_base[j] + m * HW] = v;
+    const uint32_t off = st.col_off[j] + (uint32_t)m * (uint32_t)HW * 4u;
+    buf_store(st.rsrc, (m < m_extent ? off : OOB) | (st.col_off[j] & OOB), v);
   }
 };
 

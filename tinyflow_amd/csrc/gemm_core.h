@@ -282,19 +282,27 @@ struct Across4 {
 };
 
 // ---- epilogue: plain row-major store ---------------------------------------------
+// Stores go through a buffer descriptor over this split's output: a row past
+// m_extent lies outside the buffer by itself, a column past n_extent is given an
+// out-of-range offset, and the hardware drops both -- no branch around the
+// store and 32-bit offset arithmetic only.
+__device__ inline void buf_store(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), r, (int)byte_off, 0, 0);
+}
 struct StoreRowMajor {
   float *out;
   int ld, m_extent, n_extent;
   int64_t split_stride;  // elements between the outputs of consecutive k-splits
   struct State {
-    float *base;
+    __amdgpu_buffer_rsrc_t rsrc;
   };
   template <int TN>
   __device__ inline void init(State &st, int /*n0*/, int /*lane*/, int split) const {
-    st.base = out + (int64_t)split * split_stride;
+    st.rsrc = make_rsrc(out + (int64_t)split * split_stride, (uint32_t)m_extent * (uint32_t)ld * 4u);
   }
   __device__ inline void store(const State &st, int m, int n, int /*j*/, float v) const {
-    if (m < m_extent && n < n_extent) st.base[(int64_t)m * ld + n] = v;
+    const uint32_t off = ((uint32_t)m * (uint32_t)ld + (uint32_t)n) * 4u;
+    buf_store(st.rsrc, n < n_extent ? off : OOB, v);
   }
 };
 

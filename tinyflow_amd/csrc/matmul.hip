@@ -172,8 +172,8 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   TF_REQUIRE(matC->shape[0] == M && matC->shape[1] == N, "output must be %lld x %lld", (long long)M,
              (long long)N);
   const int64_t a_bytes = numel(matA) * 4, b_bytes = numel(matB) * 4;
-  TF_REQUIRE(a_bytes < (1ll << 31) && b_bytes < (1ll << 31) && M * N < (1ll << 31),
-             "operand larger than 2 GiB is not supported");
+  TF_REQUIRE(a_bytes < (1ll << 31) && b_bytes < (1ll << 31) && M * N * 4 < (1ll << 31),
+             "operands and results of 2 GiB or more are not supported");
   hipStream_t s = stream_of(stream);
   if (M == 0 || N == 0) return 0;
   if (K == 0) return DLGpuArraySet(matC, 0.f, stream);
