@@ -138,6 +138,19 @@ def test_add_mul_and_mixed_expressions():
     assert np.array_equal(g2, 2 * v2 + 1) and np.array_equal(g3, np.ones(3))
 
 
+def test_scalar_operand_shapes():
+    """A (1,)-shaped operand (the upstream-gradient scalar) is applied as a constant:
+    the result has the other operand's shape whichever side the scalar is on.  (The
+    reference's AddOp.infer_shape returns the second operand's shape for any unequal
+    pair, autodiff.py:335-348, which under-allocates the result of ``x + scalar``.)"""
+    x, s = ad.Placeholder("x"), ad.Placeholder("s")
+    for node in (x + s, s + x, x * s, s * x):
+        shapes = {x: (4, 5), s: (1,)}
+        assert tuple(node.op.infer_shape(node, [shapes[i] for i in node.inputs], None)) == (4, 5)
+    both = x + x
+    assert tuple(both.op.infer_shape(both, [(4, 5), (4, 5)], None)) == (4, 5)
+
+
 def test_gradient_of_gradient():
     """autodiff_test.py:152-186: y = x2*x2 + x2*x3, z = dy/dx2 + dy/dx3, then dz/dx."""
     x2, x3 = ad.Variable("x2"), ad.Variable("x3")
