@@ -251,3 +251,26 @@ def test_planner_message_carries_measured_runtimes():
     conv = sum(v for k, v in by_kind.items() if k.startswith("Convolution"))
     assert conv > 0 and conv >= 0.2 * sum(by_kind.values()), by_kind
     ex.close()
+
+
+def test_swapping_adam_executor_is_bit_identical_to_the_plain_adam_executor():
+    """The swap-capable executor with the reference's optimizer (Adam): three steps with
+    swapping and recomputation give the bits of TrainExecuteAdam's plain executor."""
+    from tinyflow_amd.SwapExecute import SwapExecutor
+    from tinyflow_amd.TrainExecuteAdam import TrainExecutor
+    model, X, y = _shallow_resnet()
+    plain = TrainExecutor(model.loss, 0.001)
+    plain.init_Variable(dict(model.variables))
+    want = [[o.asnumpy() for o in plain.run({model.X: X, model.y_: y})] for _ in range(3)]
+
+    model, X, y = _shallow_resnet()
+    ex = SwapExecutor(model.loss, 0.001, swap=True, min_swap_bytes=1 << 19, prefetch_distance=4, recompute=True,
+                      optimizer="adam")
+    ex.init_Variable(dict(model.variables))
+    got = [[o.asnumpy() for o in ex.run({model.X: X, model.y_: y})] for _ in range(3)]
+    assert ex.swap_report()["offload_bytes"] > 0
+    assert abs(ex.b1t[0] - 0.9 ** 4) < 1e-12
+    for a_step, b_step in zip(want, got):
+        for a, b in zip(a_step, b_step):
+            assert a.tobytes() == b.tobytes()
+    ex.close()

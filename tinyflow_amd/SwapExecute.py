@@ -312,13 +312,28 @@ class SwapExecutor(object):
     values and swapping forward activations to pinned host memory."""
 
     def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), swap=True, min_swap_bytes=1 << 20,
-                 prefetch_distance=8, memory_budget=None, recompute=False):
+                 prefetch_distance=8, memory_budget=None, recompute=False, optimizer="sgd"):
+        """``optimizer``: "sgd" (one ``sgd_op`` per variable, as ``TrainExecute``) or "adam"
+        (one ``adam_op`` and two zero-initialised moment variables per variable with the
+        bias-correction powers advanced after every step -- the optimizer of the
+        reference's swap-capable executor, pycode/tinyflow/autodiff.py:2250-2272, 2843-2845)."""
         self.targetloss = targetloss
         self.ctx = ctx
         self.Variable_node_list = ad.get_Variable_node_list(targetloss)
         self.Variable_node_list.reverse()
         self.Variable_node_grad_list = ad.gradients(targetloss, self.Variable_node_list)
-        eval_nodes = getcomputelist(self.Variable_node_list, self.Variable_node_grad_list, learning_rate)
+        assert optimizer in ("sgd", "adam"), optimizer
+        self.optimizer = optimizer
+        self.Variable_node_to_mv = {}
+        if optimizer == "adam":
+            from . import TrainExecuteAdam as _adam
+            self.b1, self.b2, self.e = 0.9, 0.999, 0.00000001
+            self.b1t, self.b2t = [0.9], [0.999]
+            eval_nodes, self.mv, self.Variable_node_to_mv = _adam.getcomputelist(
+                self.Variable_node_list, self.Variable_node_grad_list, self.b1, self.b2, self.b1t, self.b2t,
+                self.e, learning_rate)
+        else:
+            eval_nodes = getcomputelist(self.Variable_node_list, self.Variable_node_grad_list, learning_rate)
         self.topo_order = swapsgd(ad.find_topo_sort(eval_nodes))
         self.forward_nodes = set(ad.find_topo_sort([targetloss]))
         self.swap = swap
@@ -381,7 +396,11 @@ class SwapExecutor(object):
         self.tensors = None   # re-plan on the next run
 
     def init_Variable(self, feed_dict):
-        self.Variable_node_np_value = feed_dict
+        values = dict(feed_dict)
+        for node, (m, v) in self.Variable_node_to_mv.items():   # Adam moments start at zero
+            values[m] = np.zeros(np.shape(feed_dict[node]), dtype=np.float32)
+            values[v] = np.zeros(np.shape(feed_dict[node]), dtype=np.float32)
+        self.Variable_node_np_value = values
 
     def close(self):
         self.offloader.stop()
@@ -542,6 +561,9 @@ class SwapExecutor(object):
             for n in self.release_at.get(idx, ()):
                 self._release(self.tensors[n])
         self._check_workers()
+        if self.optimizer == "adam":
+            self.b1t[0] = self.b1t[0] * self.b1
+            self.b2t[0] = self.b2t[0] * self.b2
         result = [self._on_gpu(self.tensors[self.targetloss])]
         result += [self.tensors[v].gpu for v in reversed(self.Variable_node_list)]
         if convert_to_numpy_ret_vals:
