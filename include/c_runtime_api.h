@@ -69,6 +69,13 @@ int DLArrayFree(DLArrayHandle handle);
  * ref: c_runtime_api.h:70-71, c_runtime_api.cc:130-164 */
 int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream);
 
+/* No counterpart in the reference.  Host -> device copy into an array that came from
+ * DLArrayAlloc and has not been used since (the prefetch of the swap path): only
+ * the previous life of the destination's storage has to be over, not everything
+ * that is enqueued, so the copy overlaps with the compute stream.  `stream` is a
+ * stream cell as for DLArrayCopyFromTo (not NULL); returns after the copy. */
+int DLArrayCopyIntoFresh(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream);
+
 /* ref: c_runtime_api.h:564, gpu_op.cu:4896-4898 */
 int getInt(int *intp);
 

@@ -274,3 +274,40 @@ def test_swapping_adam_executor_is_bit_identical_to_the_plain_adam_executor():
         for a, b in zip(a_step, b_step):
             assert a.tobytes() == b.tobytes()
     ex.close()
+
+
+@pytest.mark.parametrize("budget", [False, True], ids=["pool", "arena"])
+def test_copy_into_fresh_array_is_byte_exact_and_ordered_after_the_storage_s_previous_life(rt, budget):
+    """DLArrayCopyIntoFresh: a block is filled by a kernel, read back, released and
+    reallocated; the host -> device copy into the recycled storage must not overtake
+    the kernel that was still queued when the block was released.  Run on the caching
+    pool and, under a budget, on the arena (where the recycled range is found by address)."""
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(41)
+    shape = (1 << 22,)
+    side = gpu_op.create_cudaStream()
+    host = ndarray.array(rng.normal(0, 1, shape).astype(np.float32), ndarray.cpu(0))
+    if budget:
+        gpu_op.set_device_memory_limit(gpu_op.device_memory_stats()[1] + (40 << 20))   # room for two of them
+    try:
+        _copy_into_fresh_trials(rt, gpu_op, ndarray, shape, host, side)
+    finally:
+        if budget:
+            gpu_op.set_device_memory_limit(0)
+    gpu_op.destroy_cudaStream(side)
+
+
+def _copy_into_fresh_trials(rt, gpu_op, ndarray, shape, host, side):
+    for trial in range(4):
+        a = ndarray.empty(shape, rt.ctx)
+        b = ndarray.empty(shape, rt.ctx)
+        gpu_op.array_set(a, float(trial + 1), rt.stream)
+        for _ in range(8):   # a queue of work that reads a
+            gpu_op.matrix_elementwise_multiply_by_const(a, 1.0, b, rt.stream)
+        a.free_gpu()         # stream-ordered release: the kernels above still read the block
+        fresh = ndarray.empty(shape, rt.ctx)   # the same size: the pool hands the block back
+        host.copy_into_fresh(fresh, side)
+        np.testing.assert_array_equal(b.asnumpy(), np.full(shape, trial + 1, np.float32))
+        assert fresh.asnumpy().tobytes() == host.asnumpy().tobytes()
+        b.free_gpu()
+        fresh.free_gpu()

@@ -368,6 +368,55 @@ def test_swap_schedule_orders_every_transfer_around_its_uses():
         assert rel_at[n] == max(uses.get(n, [pos[n]]))
 
 
+def test_prefetch_points_placed_by_time():
+    """plan_schedule with node and copy times: every prefetch still lies between the
+    tensor's last forward and first backward use; a slower link moves the points
+    earlier; and the copies, laid out back to back on one engine with the last
+    needed last, each fit between their point and the first use."""
+    from tinyflow_amd.SwapExecute import plan_schedule
+    from tinyflow_amd.TrainExecute import getcomputelist, swapsgd
+    model, _, _ = models.build("resnet50", batch=2, image=32, n_class=10, width=4)
+    variables = list(reversed(ad.get_Variable_node_list(model.loss)))
+    topo = swapsgd(ad.find_topo_sort(getcomputelist(variables, ad.gradients(model.loss, variables), 0.1)))
+    forward = set(ad.find_topo_sort([model.loss]))
+    keep = set(variables) | {model.X, model.y_, model.loss}
+    pos = {n: i for i, n in enumerate(topo)}
+    uses = {}
+    for n in topo:
+        for inp in n.inputs:
+            uses.setdefault(inp, []).append(pos[n])
+    first_backward = min(pos[n] for n in topo if n not in forward and n.isw not in (1, 2))
+    node_seconds = 1e-3
+    clock = lambda i: i * node_seconds                     # device time at which node i starts
+
+    movable = lambda n: pos[n] % 5 == 0                    # a fifth of the values: a load the link can carry
+
+    def points(copy_seconds):
+        out, inn, _, _ = plan_schedule(topo, forward, keep, movable, 2, seconds_of=lambda n: node_seconds,
+                                       copy_seconds_of=lambda n: copy_seconds, copy_slack=1.0)
+        return ({n: t for t, ns in out.items() for n in ns}, {n: t for t, ns in inn.items() for n in ns})
+    out_fast, in_fast = points(0.5e-3)
+    out_slow, in_slow = points(2e-3)
+    assert in_fast and set(in_fast) == set(in_slow) == set(out_fast)
+    earlier = 0
+    for n in in_fast:
+        first_use = min(u for u in uses[n] if u >= first_backward)
+        for table in (in_fast, in_slow):
+            assert max(out_fast[n], first_backward - 2) < table[n] < first_use
+        assert in_slow[n] <= in_fast[n]
+        earlier += in_slow[n] < in_fast[n]
+    assert earlier > 0
+    # the slow link's copies, started when the device passes their point and run one after
+    # the other in order of need, are all in time -- unless the point is already the earliest possible
+    engine_free = 0.0
+    for n in sorted(in_slow, key=lambda n: min(u for u in uses[n] if u >= first_backward)):
+        first_use = min(u for u in uses[n] if u >= first_backward)
+        start = max(engine_free, clock(in_slow[n] + 1))
+        engine_free = start + 2e-3
+        at_floor = in_slow[n] == max(out_slow[n] + 1, first_backward - 1)
+        assert engine_free <= clock(first_use) + 1e-9 or at_floor, (n.name, engine_free, clock(first_use))
+
+
 def test_planner_wire_format_round_trip():
     """schedule_to_wire / schedule_from_wire: the planner's list format
     (reference Scheduler.py:304-331) carries the same schedule as the dicts."""

@@ -58,17 +58,21 @@ class MemoryManager(threading.Thread):
         self.stream = gpu_op.create_cudaStream()
         self.bytes_moved = 0
         self.busy_seconds = 0.0
+        self.alloc_seconds = 0.0   # part of busy_seconds spent waiting for device memory
         self.deferred = 0
         self.error = None
         self.progress = threading.Condition()
         self.pending = 0
 
-    def submit(self, tensor, to_gpu):
+    def submit(self, tensor, to_gpu, destination=None):
+        """Queue a transfer.  ``destination``: device array for a prefetch, allocated by
+        the caller at the moment of the request -- its storage was then released before
+        the request, so the copy has to wait for nothing younger than the request."""
         tensor.ready.clear()
         tensor.state = MOVING_IN if to_gpu else MOVING_OUT
         with self.progress:
             self.pending += 1
-        self.tasks.put((tensor, to_gpu))
+        self.tasks.put((tensor, to_gpu, destination))
 
     def wait_for_progress(self, timeout):
         """Block until one more queued transfer has finished (or nothing is queued)."""
@@ -84,11 +88,11 @@ class MemoryManager(threading.Thread):
             task = self.tasks.get()
             if task is None:
                 return
-            tensor, to_gpu = task
+            tensor, to_gpu, destination = task
             try:
                 t0 = time.perf_counter()
                 if to_gpu:
-                    self._swap_in(tensor)
+                    self._swap_in(tensor, destination)
                 else:
                     self._swap_out(tensor)
                 self.busy_seconds += time.perf_counter() - t0
@@ -112,26 +116,30 @@ class MemoryManager(threading.Thread):
         tensor.state = HOST
         self.bytes_moved += tensor.nbytes
 
-    def _swap_in(self, tensor):
-        arr = None
-        for _ in range(20):  # the executor thread frees memory as it advances
+    def _swap_in(self, tensor, destination=None):
+        arr = destination
+        started = time.perf_counter()
+        for _ in range(20 if arr is None else 0):  # the executor thread frees memory as it advances
             arr = ndarray.empty(tensor.shape, self.ctx)
             if not isinstance(arr, int):
                 break
             time.sleep(0.002)
+        self.alloc_seconds += time.perf_counter() - started
         if isinstance(arr, int):
             # no room yet: leave it on the host, the executor fetches it when it needs it
             self.deferred += 1
             tensor.state = HOST
             return
-        tensor.host.copyto(arr, self.stream)
+        # the array is fresh: only the previous life of its storage has to be waited for,
+        # so the copy runs beside whatever the compute stream has queued
+        tensor.host.copy_into_fresh(arr, self.stream)
         tensor.gpu = arr
         tensor.state = GPU
         self.bytes_moved += tensor.nbytes
 
 
 def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of=None, budget=None,
-                  recomputable=None):
+                  recomputable=None, seconds_of=None, copy_seconds_of=None, copy_slack=1.25):
     """Static schedule in the manner of vDNN, optionally with recomputation.
 
     Returns (swap_out, swap_in, release, recompute), each a dict ``trigger index ->
@@ -154,6 +162,13 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
       peak of the live-bytes timeline is above the budget, the candidate spanning
       the peak with the largest bytes x absence product goes (early, large
       activations first).  Without a budget every candidate moves.
+    * With ``seconds_of`` (estimated device time of a node) and ``copy_seconds_of``
+      (time to bring a tensor back over the host link) the prefetch points are placed
+      by time instead of by node count: the copies are laid out back to back on the
+      one host-to-device engine, last needed first, so that each finishes before the
+      device reaches the tensor's first backward use (each copy is given
+      ``copy_slack`` times its nominal duration); ``prefetch_distance`` then only acts
+      as the minimum distance.
     """
     pos = {n: i for i, n in enumerate(topo_order)}
     uses = {n: [] for n in topo_order}
@@ -191,7 +206,7 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
     for trigger in recompute:   # producers before consumers
         recompute[trigger].sort(key=lambda n: pos[n])
 
-    release, last_use, candidates = {}, {}, []
+    release, last_use, candidates, first_back_use = {}, {}, [], {}
     for n in movable:
         all_uses = sorted(uses[n] + extra[n])
         last = all_uses[-1] if all_uses else pos[n]
@@ -209,10 +224,48 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
         if in_at >= bwd_uses[0] or bwd_uses[0] - out_at < 2 * prefetch_distance:
             continue  # needed again too soon for a round trip to pay
         candidates.append((n, out_at, in_at))
+        first_back_use[n] = bwd_uses[0]
+    timed = seconds_of is not None and copy_seconds_of is not None
+    if timed:
+        # device time at which each node starts, if nothing ever stalls
+        clock = np.concatenate([[0.0], np.cumsum([seconds_of(n) for n in topo_order])])
+        earliest = {n: max(first_backward - 1, out_at + 1) for n, out_at, _ in candidates}
+
+        def by_time(cands, serial):
+            """Prefetch points by time; ``serial``: the copies share one engine."""
+            points, engine_free = {}, float("inf")
+            for n, out_at, in_at in sorted(cands, key=lambda c: first_back_use[c[0]], reverse=True):
+                finish = min(clock[first_back_use[n]], engine_free if serial else float("inf"))
+                start = finish - copy_slack * copy_seconds_of(n)
+                # a link that cannot keep up is not helped by asking ever earlier: the lead
+                # over the tensor's use stays within eight of its own copy times
+                start = max(start, clock[first_back_use[n]] - 8.0 * copy_slack * copy_seconds_of(n))
+                if serial:
+                    engine_free = start
+                at = int(np.searchsorted(clock, start, side="right")) - 2   # last node that ends before `start`
+                points[n] = max(min(at, in_at), earliest[n])
+            return [(n, out_at, points[n]) for n, out_at, _ in cands]
+        candidates = by_time(candidates, serial=False)
     if budget is not None:
         absent = {n: (max(u for u in uses[n] if u < first_backward), recompute_at[n]) for n in depth}
-        candidates = _fit_budget(candidates, pos, last_use, absent, nbytes_of, sum(nbytes_of(n) for n in keep),
-                                 budget, len(topo_order), prefetch_distance)
+        fit = lambda cands, forced: _fit_budget(cands, pos, last_use, absent, nbytes_of,
+                                                sum(nbytes_of(n) for n in keep), budget, len(topo_order),
+                                                prefetch_distance, forced)
+        chosen = fit(candidates, [])
+        if timed:
+            # the chosen copies queue behind each other, which moves some prefetch points
+            # forward and keeps those tensors resident longer: fit again around them
+            for _ in range(4):
+                serial = by_time(chosen, serial=True)
+                names = {c[0] for c in serial}
+                again = fit([c for c in candidates if c[0] not in names], serial)
+                chosen = again
+                if {c[0] for c in again} == names:
+                    break
+            chosen = by_time(chosen, serial=True)
+        candidates = chosen
+    elif timed:
+        candidates = by_time(candidates, serial=True)
     swap_out, swap_in = {}, {}
     for n, out_at, in_at in candidates:
         swap_out.setdefault(out_at, []).append(n)
@@ -220,11 +273,12 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
     return swap_out, swap_in, release, recompute
 
 
-def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget, steps, lag):
-    """Smallest greedy subset of ``candidates`` whose removal brings the simulated
-    footprint under ``budget``.  A swapped-out block is counted as resident until
-    ``lag`` nodes after its trigger (its copy has to finish first); ``absent`` maps a
-    recomputed value to the (release, recompute) indices between which it is gone."""
+def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget, steps, lag, forced=()):
+    """``forced`` plus the smallest greedy subset of ``candidates`` whose removal brings
+    the simulated footprint under ``budget``.  A swapped-out block is counted as
+    resident until ``lag`` nodes after its trigger (its copy has to finish first);
+    ``absent`` maps a recomputed value to the (release, recompute) indices between
+    which it is gone."""
     live = np.zeros(steps + 1, dtype=np.int64)
     for n, born in pos.items():
         if n in last_use:
@@ -233,7 +287,9 @@ def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget
     live = np.cumsum(live)[:steps] + persistent
     for n, (gone, back) in absent.items():
         live[gone + 1:back] -= nbytes_of(n)
-    chosen, remaining = [], list(candidates)
+    chosen, remaining = list(forced), list(candidates)
+    for c in forced:
+        live[c[1] + lag + 1:c[2]] -= nbytes_of(c[0])
     while remaining:
         peak = int(np.argmax(live))
         if live[peak] <= budget:
@@ -245,8 +301,7 @@ def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget
         remaining.remove(best)
         chosen.append(best)
         live[best[1] + lag + 1:best[2]] -= nbytes_of(best[0])
-    order = {c[0]: i for i, c in enumerate(candidates)}
-    return sorted(chosen, key=lambda c: order[c[0]])
+    return sorted(chosen, key=lambda c: pos[c[0]])
 
 
 def schedule_to_wire(swap_out, swap_in, release):
@@ -353,6 +408,10 @@ class SwapExecutor(object):
         self.prefetcher.start()
         self.stats = {}
         self.wire_schedule = None
+        # rate assumed for host <-> device copies when placing prefetches by time
+        # (None / 0: by node count only); PCIe 5 x16 moves ~55 GB/s in practice
+        self.host_link_bytes_per_second = 50e9
+        self.prefetch_slack = 1.25   # each prefetch is planned with this multiple of its nominal copy time
         self.measure_runtimes = False   # time every node of the next steps (waits for the device around each)
         self.node_runtime = {}          # node -> seconds, filled while measure_runtimes is set
         self._sync_cell = None
@@ -425,9 +484,17 @@ class SwapExecutor(object):
         else:
             cheap = (ad.BNForwardOp, ad.ActivationForwardOp, ad.ReluOp)
             again = (lambda n: isinstance(n.op, cheap)) if (self.swap and self.recompute) else None
+            timing = {}
+            if self.host_link_bytes_per_second:
+                # measured node times when a measured step has been run, else the estimate
+                seconds_of = (lambda n: self.node_runtime.get(n, 0.0)) if self.node_runtime \
+                    else self._estimate_seconds
+                timing = dict(seconds_of=seconds_of, copy_slack=self.prefetch_slack,
+                              copy_seconds_of=lambda n: self.tensors[n].nbytes / self.host_link_bytes_per_second)
             self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = plan_schedule(
                 self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
-                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again)
+                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again,
+                **timing)
         pos = {n: i for i, n in enumerate(self.topo_order)}
         self.uses = {n: [] for n in self.topo_order}
         for n in self.topo_order:
@@ -436,6 +503,26 @@ class SwapExecutor(object):
         self.evictable = [n for n in self.topo_order
                           if self.swap and n not in keep and not n.issgd and self.uses[n]]
         self.cursor = 0
+
+    def _estimate_seconds(self, node):
+        """Rough device time of a node for placing prefetches: a launch, the bytes the
+        node touches at 5.5 TB/s, and for a convolution or matrix product its
+        multiply-adds at 90 TFLOP/s.  Only ratios to the copy times matter."""
+        if node.isw in (1, 2):
+            return 0.0
+        moved = self.tensors[node].nbytes + sum(self.tensors[i].nbytes for i in node.inputs)
+        seconds = 5e-6 + moved / 5.5e12
+        flops = 0.0
+        if isinstance(node.op, (ad.Convolution2DForwardOp, ad.Convolution2DBackwardOp)):
+            x, w = self.tensors[node.inputs[0]].shape, self.tensors[node.inputs[1]].shape
+            y = self.tensors[node].shape if isinstance(node.op, ad.Convolution2DForwardOp) \
+                else self.tensors[node.inputs[2]].shape
+            flops = 2.0 * np.prod(y, dtype=np.float64) * w[1] * w[2] * w[3]
+        elif isinstance(node.op, ad.MatMulOp):
+            a = self.tensors[node.inputs[0]].shape
+            flops = 2.0 * np.prod(self.tensors[node].shape, dtype=np.float64) * (a[0] if node.matmul_attr_trans_A
+                                                                                 else a[1])
+        return seconds + flops / 90e12
 
     def _alloc(self, shape, what, protect=()):
         """Device array of ``shape``.  When the budget is exhausted: first wait for
@@ -451,7 +538,10 @@ class SwapExecutor(object):
             if time.perf_counter() > deadline:
                 break
             if self.offloader.pending or self.prefetcher.pending:
+                waited = time.perf_counter()
                 self.offloader.wait_for_progress(0.05)
+                self.stats["alloc_wait_seconds"] = (self.stats.get("alloc_wait_seconds", 0.0)
+                                                    + time.perf_counter() - waited)
                 continue
             victim = self._pick_victim(protect)
             if victim is None:
@@ -481,7 +571,10 @@ class SwapExecutor(object):
     def _on_gpu(self, tensor, protect=()):
         """Device array of a tensor, fetching it back first if it was swapped out."""
         if tensor.state in (MOVING_OUT, MOVING_IN):
+            waited = time.perf_counter()
             tensor.ready.wait()
+            self.stats["transfer_wait_seconds"] = (self.stats.get("transfer_wait_seconds", 0.0)
+                                                   + time.perf_counter() - waited)
             self._check_workers()
         if tensor.state == FREED and tensor.node.inputs and tensor.node.isw not in (1, 2):
             self._recompute(tensor.node, self._handles)   # released and not brought back: recompute
@@ -557,7 +650,8 @@ class SwapExecutor(object):
                 if tn.state == MOVING_OUT:
                     tn.ready.wait()
                 if tn.state == HOST:
-                    self.prefetcher.submit(tn, True)
+                    room = ndarray.empty(tn.shape, self.ctx)   # None: the worker asks again later
+                    self.prefetcher.submit(tn, True, None if isinstance(room, int) else room)
             for n in self.release_at.get(idx, ()):
                 self._release(self.tensors[n])
         self._check_workers()
@@ -604,7 +698,12 @@ class SwapExecutor(object):
         """Bytes moved and busy time of the two copy workers since construction."""
         return {"offload_bytes": self.offloader.bytes_moved, "offload_seconds": self.offloader.busy_seconds,
                 "prefetch_bytes": self.prefetcher.bytes_moved, "prefetch_seconds": self.prefetcher.busy_seconds,
+                "prefetch_alloc_seconds": self.prefetcher.alloc_seconds,
                 "passive_swap_in": self.stats.get("passive_swap_in", 0),
                 "passive_swap_out": self.stats.get("passive_swap_out", 0),
                 "passive_bytes": self.stats.get("passive_bytes", 0),
-                "prefetch_deferred": self.prefetcher.deferred, "recomputed": self.stats.get("recomputed", 0)}
+                "prefetch_deferred": self.prefetcher.deferred, "recomputed": self.stats.get("recomputed", 0),
+                # host time the step spent blocked: on memory (waiting for offloads to free
+                # blocks) and on operands whose transfer had not finished
+                "alloc_wait_seconds": self.stats.get("alloc_wait_seconds", 0.0),
+                "transfer_wait_seconds": self.stats.get("transfer_wait_seconds", 0.0)}

@@ -49,8 +49,25 @@ struct Runtime {
     bool retired = false;                        // budget changed: serve no new requests
     std::map<size_t, size_t> free_by_off;        // offset -> length
     std::multimap<size_t, size_t> free_by_len;   // length -> offset
+    // release fences by address: non-overlapping segments covering the arena, each with the
+    // fence of the last release that touched it (free ranges coalesce, their histories must not:
+    // a merged range would inherit its youngest neighbour's fence)
+    struct Seg { size_t len; uint64_t fence; };
+    std::map<size_t, Seg> fence_seg;             // offset -> segment
     std::unordered_map<void *, size_t> used;     // pointer -> length
   } arena;
+  // Release fences.  Every device block remembers the number of the fence that was
+  // recorded, on the kernel-running stream, when its storage was last given back:
+  // all kernels that could still touch the storage were enqueued before that
+  // fence.  Fences live in a ring of events; a slot that has been reused holds a
+  // later fence of the same stream, which is just as safe to wait for.
+  static constexpr int kFenceRing = 1024;
+  static constexpr uint64_t kNoFence = 0;                  // storage never handed back since it came from HIP
+  static constexpr uint64_t kConservative = ~(uint64_t)0;  // no single stream to fence on: wait for all
+  hipEvent_t fence_ring[kFenceRing] = {};
+  uint64_t fence_count = 0;
+  std::unordered_map<void *, uint64_t> pool_fence;   // cached / handed-out pool block -> fence of its last release
+  std::unordered_map<void *, uint64_t> block_fence;  // handed-out device block -> fence to honour before reuse
   std::vector<StreamRec> streams;
   bool sync_ops = false;
   int cus = 0;
@@ -82,7 +99,12 @@ void release_cached(Runtime::Pool &p, bool device, size_t need, size_t limit) {
   while (!p.free_blocks.empty()) {
     if (limit != 0 && p.reserved + need <= limit) break;
     auto it = std::prev(p.free_blocks.end());
-    if (device) (void)hipFree(it->second); else (void)hipHostFree(it->second);
+    if (device) {
+      (void)hipFree(it->second);
+      rt().pool_fence.erase(it->second);
+    } else {
+      (void)hipHostFree(it->second);
+    }
     p.reserved -= it->first;
     p.block_size.erase(it->second);
     p.free_blocks.erase(it);
@@ -104,10 +126,56 @@ void arena_insert_free(Runtime::Arena &a, size_t off, size_t len) {
   a.free_by_len.emplace(len, off);
 }
 
-void *arena_alloc(Runtime::Arena &a, size_t want) {
+// Fence numbers grow along the one stream they are recorded on, so the later of two is the larger.
+uint64_t later_fence(uint64_t x, uint64_t y) { return x > y ? x : y; }
+
+// Stamps [off, off + len) with `fence`, splitting the segments it overlaps.
+void arena_set_fence(Runtime::Arena &a, size_t off, size_t len, uint64_t fence) {
+  const size_t end = off + len;
+  auto it = a.fence_seg.upper_bound(off);
+  if (it != a.fence_seg.begin()) --it;
+  while (it != a.fence_seg.end() && it->first < end) {
+    const size_t s_off = it->first, s_end = it->first + it->second.len;
+    const uint64_t s_fence = it->second.fence;
+    if (s_end <= off) {
+      ++it;
+      continue;
+    }
+    it = a.fence_seg.erase(it);
+    if (s_off < off) a.fence_seg[s_off] = {off - s_off, s_fence};          // part in front survives
+    if (s_end > end) it = a.fence_seg.emplace(end, Runtime::Arena::Seg{s_end - end, s_fence}).first;  // part behind
+  }
+  auto mine = a.fence_seg.emplace(off, Runtime::Arena::Seg{len, fence}).first;
+  // fold equal neighbours together so the map stays as small as the arena's block structure
+  auto next = std::next(mine);
+  if (next != a.fence_seg.end() && next->second.fence == fence && mine->first + mine->second.len == next->first) {
+    mine->second.len += next->second.len;
+    a.fence_seg.erase(next);
+  }
+  if (mine != a.fence_seg.begin()) {
+    auto prev = std::prev(mine);
+    if (prev->second.fence == fence && prev->first + prev->second.len == mine->first) {
+      prev->second.len += mine->second.len;
+      a.fence_seg.erase(mine);
+    }
+  }
+}
+
+// Latest fence among the segments that [off, off + len) overlaps.
+uint64_t arena_fence_of(const Runtime::Arena &a, size_t off, size_t len) {
+  uint64_t fence = Runtime::kNoFence;
+  auto it = a.fence_seg.upper_bound(off);
+  if (it != a.fence_seg.begin()) --it;
+  for (; it != a.fence_seg.end() && it->first < off + len; ++it)
+    if (it->first + it->second.len > off) fence = later_fence(fence, it->second.fence);
+  return fence;
+}
+
+void *arena_alloc(Runtime::Arena &a, size_t want, uint64_t *fence) {
   auto it = a.free_by_len.lower_bound(want);  // best fit
   if (it == a.free_by_len.end()) return nullptr;
   const size_t len = it->first, off = it->second;
+  *fence = arena_fence_of(a, off, want);
   arena_erase_free(a, off, len);
   if (len > want) arena_insert_free(a, off + want, len - want);
   void *ptr = a.base + off;
@@ -116,13 +184,15 @@ void *arena_alloc(Runtime::Arena &a, size_t want) {
   return ptr;
 }
 
-// Returns false when `ptr` does not belong to the arena.
-bool arena_free(Runtime::Arena &a, void *ptr) {
+// Returns false when `ptr` does not belong to the arena.  `fence` is the release
+// fence of the block.
+bool arena_free(Runtime::Arena &a, void *ptr, uint64_t fence) {
   auto it = a.used.find(ptr);
   if (it == a.used.end()) return false;
   size_t off = (size_t)((char *)ptr - a.base), len = it->second;
   a.used_bytes -= len;
   a.used.erase(it);
+  arena_set_fence(a, off, len, fence);
   auto next = a.free_by_off.lower_bound(off);
   if (next != a.free_by_off.end() && next->first == off + len) {  // merge with the range behind
     const size_t nlen = next->second;
@@ -205,6 +275,34 @@ void arena_open(Runtime &r) {
   r.arena.base = (char *)base;
   r.arena.size = size;
   arena_insert_free(r.arena, 0, size);
+  r.arena.fence_seg[0] = {size, Runtime::kNoFence};
+}
+
+// Records a release fence on the one stream that runs kernels and returns its
+// number; kConservative when there is no such single stream (none yet, or several).
+// Called with the lock held.
+uint64_t record_release_fence(Runtime &r) {
+  hipStream_t only = nullptr;
+  int kernel_streams = 0;
+  for (auto &rec : r.streams)
+    if (rec.runs_kernels) {
+      only = rec.stream;
+      ++kernel_streams;
+    }
+  if (kernel_streams != 1) return Runtime::kConservative;
+  const uint64_t number = r.fence_count + 1;
+  hipEvent_t &ev = r.fence_ring[number % Runtime::kFenceRing];
+  if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+    ev = nullptr;
+    (void)hipGetLastError();
+    return Runtime::kConservative;
+  }
+  if (hipEventRecord(ev, only) != hipSuccess) {
+    (void)hipGetLastError();
+    return Runtime::kConservative;
+  }
+  r.fence_count = number;
+  return number;
 }
 
 void *device_alloc(size_t bytes) {
@@ -214,24 +312,52 @@ void *device_alloc(size_t bytes) {
   if (r.dev_limit != 0) {
     if (!r.arena.base) arena_open(r);
     if (r.arena.base && !r.arena.retired) {
-      void *ptr = arena_alloc(r.arena, round_size(bytes));
+      uint64_t fence = Runtime::kNoFence;
+      void *ptr = arena_alloc(r.arena, round_size(bytes), &fence);
       if (ptr) {
+        r.block_fence[ptr] = fence;
         const size_t total = r.dev.in_use + r.arena.used_bytes;
         if (total > r.dev.peak_in_use) r.dev.peak_in_use = total;
       }
       return ptr;
     }
   }
-  return pool_alloc(r.dev, bytes, true, r.dev_limit);
+  void *ptr = pool_alloc(r.dev, bytes, true, r.dev_limit);
+  if (ptr) {
+    auto it = r.pool_fence.find(ptr);
+    r.block_fence[ptr] = it == r.pool_fence.end() ? Runtime::kNoFence : it->second;
+  }
+  return ptr;
 }
 void device_free(void *p) {
   if (!p) return;
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
-  if (r.arena.base && arena_free(r.arena, p)) return;
+  if (r.block_fence.erase(p) == 0) return;  // not a block handed out by device_alloc
+  const uint64_t fence = record_release_fence(r);
+  if (r.arena.base && arena_free(r.arena, p, fence)) return;
+  r.pool_fence[p] = fence;
   pool_free(r.dev, p);
   // a pool block returned while a budget is active must not linger in the cache
   if (r.dev_limit != 0 && r.arena.base) release_cached(r.dev, true, 0, 0);
+}
+
+// Makes `s` wait until the previous life of the storage behind `ptr` (a block handed
+// out by device_alloc and not used since) is over.  Returns 0, or 1 when no fence
+// is known and the caller has to wait for all kernel streams instead.
+int wait_for_previous_life(void *ptr, hipStream_t s) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  auto it = r.block_fence.find(ptr);
+  if (it == r.block_fence.end() || it->second == Runtime::kConservative) return 1;
+  if (it->second == Runtime::kNoFence) return 0;
+  // a slot reused since then holds a later fence of the same stream
+  hipEvent_t ev = r.fence_ring[it->second % Runtime::kFenceRing];
+  if (!ev || hipStreamWaitEvent(s, ev, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return 1;
+  }
+  return 0;
 }
 void *pinned_alloc(size_t bytes) {
   Runtime &r = rt();
@@ -404,6 +530,26 @@ extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamH
   // Host memory must be readable / reusable on return.  A device-to-device copy
   // is only ever observed by later stream-ordered work, so it stays asynchronous.
   if (kind != hipMemcpyDeviceToDevice || sync_every_op()) TF_HIP(hipStreamSynchronize(s));
+  return 0;
+}
+
+// Host -> device copy into an array that came from DLArrayAlloc and has not been
+// used since (no counterpart in the reference; the prefetch of the swap path).
+// DLArrayCopyFromTo must assume that kernels already enqueued may still read the
+// destination and therefore waits for all of them; here only the previous life of
+// the destination's storage has to be over, which is known from the fence recorded
+// when that storage was released -- usually long ago, so the copy overlaps with
+// whatever the compute stream is doing.  Returns after the copy has completed.
+extern "C" int DLArrayCopyIntoFresh(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
+  TF_REQUIRE(from && to && from->data && to->data && stream, "null argument");
+  TF_REQUIRE(from->ctx.device_type == kCPU && to->ctx.device_type == kGPU, "host to device only");
+  const size_t bytes = array_bytes(from);
+  TF_REQUIRE(bytes == array_bytes(to), "size mismatch (%zu vs %zu bytes)", bytes, array_bytes(to));
+  if (bytes == 0) return 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(*reinterpret_cast<void **>(stream));
+  if (wait_for_previous_life(to->data, s) != 0 && wait_for_other_streams(s) != 0) return -1;
+  TF_HIP(hipMemcpyAsync(to->data, from->data, bytes, hipMemcpyHostToDevice, s));
+  TF_HIP(hipStreamSynchronize(s));
   return 0;
 }
 

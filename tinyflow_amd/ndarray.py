@@ -147,6 +147,13 @@ class NDArray(object):
         check_call(_LIB.DLArrayCopyFromTo(self.handle, target.handle, cudaStream))
         return target
 
+    def copy_into_fresh(self, target, cudaStream):
+        """Host -> device copy into ``target``, a device array that was just allocated and
+        has not been used yet: waits only for the previous life of its storage, not
+        for everything enqueued (the prefetch of the swap path)."""
+        check_call(_LIB.DLArrayCopyIntoFresh(self.handle, target.handle, cudaStream))
+        return target
+
 
 def empty(shape, ctx=cpu(0)):
     """Uninitialised array; returns the wanted byte count (int) when out of memory."""
