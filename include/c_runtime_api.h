@@ -76,6 +76,12 @@ int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle strea
  * stream cell as for DLArrayCopyFromTo (not NULL); returns after the copy. */
 int DLArrayCopyIntoFresh(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream);
 
+/* No counterpart in the reference.  Call right after DLArrayAlloc on an array that
+ * DLArrayCopyIntoFresh will fill later: records, now, the fence that covers the
+ * last release of the array's storage, so that the copy waits for nothing enqueued
+ * after this call.  Without it DLArrayCopyIntoFresh waits like DLArrayCopyFromTo. */
+int DLArrayPrepareFresh(DLArrayHandle arr);
+
 /* ref: c_runtime_api.h:564, gpu_op.cu:4896-4898 */
 int getInt(int *intp);
 

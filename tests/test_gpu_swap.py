@@ -306,6 +306,8 @@ def _copy_into_fresh_trials(rt, gpu_op, ndarray, shape, host, side):
             gpu_op.matrix_elementwise_multiply_by_const(a, 1.0, b, rt.stream)
         a.free_gpu()         # stream-ordered release: the kernels above still read the block
         fresh = ndarray.empty(shape, rt.ctx)   # the same size: the pool hands the block back
+        if trial % 2 == 0:
+            fresh.prepare_fresh()   # with the fence: waits for the queue above only; without: for everything
         host.copy_into_fresh(fresh, side)
         np.testing.assert_array_equal(b.asnumpy(), np.full(shape, trial + 1, np.float32))
         assert fresh.asnumpy().tobytes() == host.asnumpy().tobytes()

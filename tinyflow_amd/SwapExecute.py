@@ -650,8 +650,12 @@ class SwapExecutor(object):
                 if tn.state == MOVING_OUT:
                     tn.ready.wait()
                 if tn.state == HOST:
-                    room = ndarray.empty(tn.shape, self.ctx)   # None: the worker asks again later
-                    self.prefetcher.submit(tn, True, None if isinstance(room, int) else room)
+                    room = ndarray.empty(tn.shape, self.ctx)
+                    if isinstance(room, int):
+                        room = None   # no room now: the worker asks again later
+                    else:
+                        room.prepare_fresh()
+                    self.prefetcher.submit(tn, True, room)
             for n in self.release_at.get(idx, ()):
                 self._release(self.tensors[n])
         self._check_workers()

@@ -147,6 +147,12 @@ class NDArray(object):
         check_call(_LIB.DLArrayCopyFromTo(self.handle, target.handle, cudaStream))
         return target
 
+    def prepare_fresh(self):
+        """Call right after allocating a device array that ``copy_into_fresh`` will fill
+        later: the copy then waits for nothing enqueued after this call."""
+        check_call(_LIB.DLArrayPrepareFresh(self.handle))
+        return self
+
     def copy_into_fresh(self, target, cudaStream):
         """Host -> device copy into ``target``, a device array that was just allocated and
         has not been used yet: waits only for the previous life of its storage, not
