@@ -325,7 +325,9 @@ def main():
         from tinyflow_amd.SwapExecute import SwapExecutor
         limit = int(args.mem_limit_gb * (1 << 30))
         gpu_op.set_device_memory_limit(limit)
-        ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=int(0.95 * limit), prefetch_distance=12,
+        # planned for the whole budget; a step that has to evict on demand makes the
+        # executor plan for 3 % less (which the warm-up steps absorb)
+        ex = SwapExecutor(model.loss, 0.01, swap=True, memory_budget=limit, prefetch_distance=12,
                           recompute=not args.no_recompute)
     else:
         ex = TrainExecutor(model.loss, 0.01, fuse_bn_relu=args.fuse_bn_relu)
@@ -457,7 +459,7 @@ def main():
         "fused_bn_relu": fused,
     }
     if swap_before:
-        moved = {k: swap_after[k] - swap_before[k] for k in swap_after}
+        moved = {k: swap_after[k] - swap_before[k] for k in swap_after if k != "planned_budget_bytes"}
         reserved, _, peak = swap_mem
         result["swap"] = {
             "device_budget_bytes": int(args.mem_limit_gb * (1 << 30)), "peak_in_use_bytes": peak,
@@ -470,6 +472,8 @@ def main():
                                    / wall / 1e9,
             "passive_swap_in": moved["passive_swap_in"], "passive_swap_out": moved["passive_swap_out"],
             "recomputed_per_step": moved["recomputed"] / args.steps,
+            "planned_budget_bytes": swap_after["planned_budget_bytes"],
+            "budget_reductions_in_timed_steps": moved["budget_reductions"],
         }
         ex.close()
     if not args.no_cpu_baseline:

@@ -412,6 +412,8 @@ class SwapExecutor(object):
         # (None / 0: by node count only); PCIe 5 x16 moves ~55 GB/s in practice
         self.host_link_bytes_per_second = 50e9
         self.prefetch_slack = 1.25   # each prefetch is planned with this multiple of its nominal copy time
+        self.adapt_budget = True     # lower the planned budget when a step had to evict on demand
+        self._evictions_seen = 0
         self.measure_runtimes = False   # time every node of the next steps (waits for the device around each)
         self.node_runtime = {}          # node -> seconds, filled while measure_runtimes is set
         self._sync_cell = None
@@ -473,28 +475,9 @@ class SwapExecutor(object):
             if node not in shapes:
                 shapes[node] = tuple(node.op.infer_shape(node, [shapes[i] for i in node.inputs], self.cudnnHandle))
         self.tensors = {node: _Tensor(node, shapes[node]) for node in self.topo_order}
-        keep = set(n for n in self.topo_order if n.isw in (1, 2)) | {self.targetloss} | self.keep_values
-        self.keep = keep
-        big = lambda n: self.swap and self.tensors[n].nbytes >= self.min_swap_bytes
-        self.recompute_at = {}
-        if self.wire_schedule is not None:
-            by_node = [{t: [self.topo_order[i] for i in ids if self.topo_order[i] not in keep]
-                        for t, ids in table.items()} for table in self.wire_schedule]
-            self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = by_node
-        else:
-            cheap = (ad.BNForwardOp, ad.ActivationForwardOp, ad.ReluOp)
-            again = (lambda n: isinstance(n.op, cheap)) if (self.swap and self.recompute) else None
-            timing = {}
-            if self.host_link_bytes_per_second:
-                # measured node times when a measured step has been run, else the estimate
-                seconds_of = (lambda n: self.node_runtime.get(n, 0.0)) if self.node_runtime \
-                    else self._estimate_seconds
-                timing = dict(seconds_of=seconds_of, copy_slack=self.prefetch_slack,
-                              copy_seconds_of=lambda n: self.tensors[n].nbytes / self.host_link_bytes_per_second)
-            self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = plan_schedule(
-                self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
-                nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again,
-                **timing)
+        self.keep = set(n for n in self.topo_order if n.isw in (1, 2)) | {self.targetloss} | self.keep_values
+        self._plan()
+        keep = self.keep
         pos = {n: i for i, n in enumerate(self.topo_order)}
         self.uses = {n: [] for n in self.topo_order}
         for n in self.topo_order:
@@ -503,6 +486,30 @@ class SwapExecutor(object):
         self.evictable = [n for n in self.topo_order
                           if self.swap and n not in keep and not n.issgd and self.uses[n]]
         self.cursor = 0
+
+    def _plan(self):
+        """(Re)builds the swap / release / recomputation tables for the current budget."""
+        keep = self.keep
+        big = lambda n: self.swap and self.tensors[n].nbytes >= self.min_swap_bytes
+        self.recompute_at = {}
+        if self.wire_schedule is not None:
+            by_node = [{t: [self.topo_order[i] for i in ids if self.topo_order[i] not in keep]
+                        for t, ids in table.items()} for table in self.wire_schedule]
+            self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = by_node
+            return
+        cheap = (ad.BNForwardOp, ad.ActivationForwardOp, ad.ReluOp)
+        again = (lambda n: isinstance(n.op, cheap)) if (self.swap and self.recompute) else None
+        timing = {}
+        if self.host_link_bytes_per_second:
+            # measured node times when a measured step has been run, else the estimate
+            seconds_of = (lambda n: self.node_runtime.get(n, 0.0)) if self.node_runtime \
+                else self._estimate_seconds
+            timing = dict(seconds_of=seconds_of, copy_slack=self.prefetch_slack,
+                          copy_seconds_of=lambda n: self.tensors[n].nbytes / self.host_link_bytes_per_second)
+        self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = plan_schedule(
+            self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
+            nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again,
+            **timing)
 
     def _estimate_seconds(self, node):
         """Rough device time of a node for placing prefetches: a launch, the bytes the
@@ -659,6 +666,7 @@ class SwapExecutor(object):
             for n in self.release_at.get(idx, ()):
                 self._release(self.tensors[n])
         self._check_workers()
+        self._adapt_budget()
         if self.optimizer == "adam":
             self.b1t[0] = self.b1t[0] * self.b1
             self.b2t[0] = self.b2t[0] * self.b2
@@ -667,6 +675,20 @@ class SwapExecutor(object):
         if convert_to_numpy_ret_vals:
             return [r.asnumpy() for r in result]
         return result
+
+    def _adapt_budget(self):
+        """The schedule is planned for ``memory_budget``; what the plan does not model
+        (scratch of the operators, fragmentation) can make a step that fits on paper
+        evict on demand.  A step that had to do so lowers the planned budget by 3 % and
+        plans again, at most ten times; steps that fit leave the plan alone."""
+        evictions = self.stats.get("passive_swap_out", 0) + self.stats.get("passive_swap_in", 0)
+        happened = evictions > self._evictions_seen
+        self._evictions_seen = evictions
+        if (happened and self.adapt_budget and self.memory_budget and self.wire_schedule is None
+                and self.stats.get("budget_reductions", 0) < 10):
+            self.memory_budget = int(self.memory_budget * 0.97)
+            self.stats["budget_reductions"] = self.stats.get("budget_reductions", 0) + 1
+            self._plan()
 
     def _recompute(self, node, handles):
         """Evaluate ``node`` again from its inputs (a planner released its value and
@@ -709,5 +731,6 @@ class SwapExecutor(object):
                 "prefetch_deferred": self.prefetcher.deferred, "recomputed": self.stats.get("recomputed", 0),
                 # host time the step spent blocked: on memory (waiting for offloads to free
                 # blocks) and on operands whose transfer had not finished
+                "planned_budget_bytes": self.memory_budget, "budget_reductions": self.stats.get("budget_reductions", 0),
                 "alloc_wait_seconds": self.stats.get("alloc_wait_seconds", 0.0),
                 "transfer_wait_seconds": self.stats.get("transfer_wait_seconds", 0.0)}
