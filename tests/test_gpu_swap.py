@@ -313,3 +313,44 @@ def _copy_into_fresh_trials(rt, gpu_op, ndarray, shape, host, side):
         assert fresh.asnumpy().tobytes() == host.asnumpy().tobytes()
         b.free_gpu()
         fresh.free_gpu()
+
+
+def test_planned_budget_adapts_when_a_step_has_to_evict():
+    """A plan made for more memory than the device limit grants runs into on-demand
+    evictions; the executor then plans for 3 % less per offending step until the steps
+    fit, and every step -- evicting or not -- gives the plain executor's bits."""
+    from tinyflow_amd import gpu_op
+    from tinyflow_amd.SwapExecute import SwapExecutor
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    model, X, y = _shallow_resnet(batch=32, image=96, width=16)
+    plain = TrainExecutor(model.loss, 0.01)
+    plain.init_Variable(dict(model.variables))
+    steps = 8
+    want = [plain.run({model.X: X, model.y_: y})[0].asnumpy().tobytes() for _ in range(steps)]
+    del plain
+    # what the released-early executor needs at its peak, then a limit 25 % below it
+    gpu_op.set_device_memory_limit(0)
+    try:
+        model, X, y = _shallow_resnet(batch=32, image=96, width=16)
+        base = gpu_op.device_memory_stats(reset_peak=True)[1]
+        probe = SwapExecutor(model.loss, 0.01, swap=False)
+        probe.init_Variable(dict(model.variables))
+        probe.run({model.X: X, model.y_: y})[0].asnumpy()
+        need = gpu_op.device_memory_stats()[2] - base
+        probe.close()
+        del probe
+        base = gpu_op.device_memory_stats()[1]
+        limit = int(0.75 * need)
+        gpu_op.set_device_memory_limit(base + limit)
+        model, X, y = _shallow_resnet(batch=32, image=96, width=16)
+        ex = SwapExecutor(model.loss, 0.01, swap=True, min_swap_bytes=1 << 16, prefetch_distance=4,
+                          memory_budget=int(1.3 * limit))          # a plan that is too optimistic
+        ex.init_Variable(dict(model.variables))
+        got = [ex.run({model.X: X, model.y_: y})[0].asnumpy().tobytes() for _ in range(steps)]
+        rep = ex.swap_report()
+        assert got == want
+        assert rep["passive_swap_out"] > 0 and rep["budget_reductions"] > 0
+        assert rep["planned_budget_bytes"] < int(1.3 * limit)
+        ex.close()
+    finally:
+        gpu_op.set_device_memory_limit(0)
