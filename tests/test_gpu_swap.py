@@ -224,10 +224,10 @@ def test_planner_message_carries_measured_runtimes():
     the measuring step itself still gives the plain executor's bits."""
     from tinyflow_amd.SwapExecute import SwapExecutor
     from tinyflow_amd.TrainExecute import TrainExecutor
-    model, X, y = _shallow_resnet()
-    plain = TrainExecutor(model.loss, 0.01)
-    plain.init_Variable(dict(model.variables))
-    want = [o.asnumpy() for o in plain.run({model.X: X, model.y_: y})]
+    pmodel, pX, py = _shallow_resnet()
+    plain = TrainExecutor(pmodel.loss, 0.01)
+    plain.init_Variable(dict(pmodel.variables))
+    want = [o.asnumpy() for o in plain.run({pmodel.X: pX, pmodel.y_: py})]
 
     model, X, y = _shallow_resnet()
     ex = SwapExecutor(model.loss, 0.01, swap=False)
@@ -239,6 +239,12 @@ def test_planner_message_carries_measured_runtimes():
         assert a.tobytes() == b.tobytes()
     msg = ex.planner_message()
     assert len(msg) == len(ex.topo_order)
+    # the measured times can also place the prefetches of the built-in schedule
+    ex.replan()
+    again = [o.asnumpy() for o in ex.run({model.X: X, model.y_: y})]
+    second = [o.asnumpy() for o in plain.run({pmodel.X: pX, pmodel.y_: py})]
+    for a, b in zip(second, again):
+        assert a.tobytes() == b.tobytes()
     by_kind = {}
     for node, (tensors, inputs, name, op_id, flag, _, runtime) in zip(ex.topo_order, msg):
         if node.isw in (1, 2):

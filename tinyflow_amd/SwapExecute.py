@@ -487,6 +487,12 @@ class SwapExecutor(object):
                           if self.swap and n not in keep and not n.issgd and self.uses[n]]
         self.cursor = 0
 
+    def replan(self):
+        """Builds the schedule again, e.g. after a step run with ``measure_runtimes`` so
+        that the prefetch points use measured node times instead of the estimate."""
+        assert self.tensors is not None, "run one step first: shapes are inferred there"
+        self._plan()
+
     def _plan(self):
         """(Re)builds the swap / release / recomputation tables for the current budget."""
         keep = self.keep
