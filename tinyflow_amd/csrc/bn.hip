@@ -10,23 +10,27 @@
 //   single pass: forward reads x and writes y (8 B/element), backward reads x, dy
 //   and writes dx (12 B/element).  Lanes of a wave read 64 consecutive columns,
 //   so every access is a full 256-byte line.
-// spatial mode: one statistic per channel over (N,H,W).  Two passes: per-(channel,
-//   image-chunk) partial sums in fp64, then a normalise pass that first folds the
-//   partials of its channel in a fixed order (12 B/element forward, 20 backward).
+// spatial mode: one statistic per channel over (N,H,W).  Three kernels: per-(channel,
+//   image-chunk) partial sums (fp32 per lane, fp64 across lanes and chunks), a tiny
+//   one that folds the chunks of every channel in a fixed order, and a streaming
+//   normalise pass over the flat tensor (12 B/element forward, 20 backward).
 //
 // Saved statistics protocol (as the reference): forward allocates mean and
 // inverse-std buffers and publishes them through *mean_p / *Variance_p; backward
 // consumes and releases them.
+#include "gemm_core.h"
 #include "internal.h"
 
 #include <type_traits>
 
 using namespace tf;
+using tf::gemm::FastDiv;
 
 namespace {
 
 constexpr int kThreads = 256;
 constexpr float kEps = 1e-5f;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- per-activation
 
@@ -174,41 +178,71 @@ __device__ inline void block_sum2(double &a, double &b, double (*smem)[2]) {
   }
 }
 
+// One unit of the spatial kernels: a 16-byte vector (feature maps whose size is a
+// multiple of 4) or a single float.
+template <bool VEC>
+struct Unit;
+template <>
+struct Unit<true> {
+  static constexpr int W = 4;
+  static __device__ inline void load(const float *p, float (&v)[4]) {
+    const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  static __device__ inline void store(float *p, const float (&v)[4]) {
+    const f32x4 t = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4 *>(p) = t;
+  }
+};
+template <>
+struct Unit<false> {
+  static constexpr int W = 1;
+  static __device__ inline void load(const float *p, float (&v)[1]) { v[0] = *p; }
+  static __device__ inline void store(float *p, const float (&v)[1]) { *p = v[0]; }
+};
+
 // x viewed as [N, C, HW]; block (c, chunk) sums images [chunk*ipc, ...) of channel c.
-// FWD: partial = (sum x, sum x^2); BWD: partial = (sum dy, sum dy*xhat)
-template <bool BWD>
+// FWD: partial = (sum x, sum x^2); BWD: partial = (sum dy, sum dy*xhat).
+// The (image, pixel) pairs of a chunk are walked as one flat index so that small
+// feature maps (7x7) keep all lanes busy; VEC: 16-byte loads when HW is a multiple
+// of 4.  Lanes accumulate in fp32 (a few hundred terms each), the block and the
+// chunks are combined in fp64.
+template <bool BWD, bool VEC>
 __global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ dy,
                                                                 const float *__restrict__ save_mean,
                                                                 const float *__restrict__ save_istd,
                                                                 double *__restrict__ partial, int N, int C,
-                                                                int HW, int images_per_chunk) {
+                                                                int HW, int images_per_chunk, FastDiv div_row) {
   __shared__ double smem[4][2];
   const int c = blockIdx.x;
   const int n0 = blockIdx.y * images_per_chunk;
   int n1 = n0 + images_per_chunk;
   if (n1 > N) n1 = N;
   const float mean = BWD ? save_mean[c] : 0.f, istd = BWD ? save_istd[c] : 0.f;
+  constexpr int W = Unit<VEC>::W;
+  const uint32_t row_units = (uint32_t)HW / W;                 // div_row divides by this
+  const uint32_t total = (uint32_t)(n1 - n0) * row_units;
   float a0 = 0.f, b0 = 0.f;
-  double a = 0.0, b = 0.0;
-  for (int n = n0; n < n1; ++n) {
-    const int64_t row = ((int64_t)n * C + c) * HW;
-    a0 = 0.f;
-    b0 = 0.f;
-    for (int i = threadIdx.x; i < HW; i += kThreads) {
-      const float xv = x[row + i];
+  for (uint32_t idx = threadIdx.x; idx < total; idx += kThreads) {
+    uint32_t img, unit;
+    div_row.divmod(idx, img, unit);
+    const int64_t at = ((int64_t)(n0 + (int)img) * C + c) * HW + (int64_t)unit * W;
+    float xv[W], gv[W] = {};
+    Unit<VEC>::load(x + at, xv);
+    if (BWD) Unit<VEC>::load(dy + at, gv);
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
       if (BWD) {
-        const float g = dy[row + i];
-        a0 += g;
-        b0 += g * ((xv - mean) * istd);
+        a0 += gv[k];
+        b0 += gv[k] * ((xv[k] - mean) * istd);
       } else {
-        a0 += xv;
-        b0 += xv * xv;
+        a0 += xv[k];
+        b0 += xv[k] * xv[k];
       }
     }
-    a += (double)a0;  // per-image fp32 partials, accumulated across images in fp64
-    b += (double)b0;
   }
+  double a = (double)a0, b = (double)b0;
   block_sum2(a, b, smem);
   if (threadIdx.x == 0) {
     partial[((int64_t)blockIdx.y * C + c) * 2 + 0] = a;
@@ -216,54 +250,79 @@ __global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__
   }
 }
 
-// one block per (n, c) row of HW elements; folds the channel's partials first
-__global__ __launch_bounds__(kThreads) void bn_sp_forward_apply_kernel(const float *__restrict__ x,
-                                                                      float *__restrict__ y,
-                                                                      const double *__restrict__ partial,
-                                                                      float *__restrict__ save_mean,
-                                                                      float *__restrict__ save_istd, int N,
-                                                                      int C, int HW, int chunks) {
-  const int c = blockIdx.x % C;
+// Folds the chunk partials of every channel, in chunk order, into the two floats
+// the apply pass needs: forward (mean, 1/sqrt(var + eps)), which are also the saved
+// statistics; backward (sum dy, sum dy*xhat).
+template <bool BWD>
+__global__ __launch_bounds__(kThreads) void bn_sp_finish_kernel(const double *__restrict__ partial,
+                                                               float *__restrict__ out0, float *__restrict__ out1,
+                                                               int N, int C, int HW, int chunks) {
+  const int c = blockIdx.x * kThreads + threadIdx.x;
+  if (c >= C) return;
   double s = 0.0, q = 0.0;
   for (int k = 0; k < chunks; ++k) {
     s += partial[((int64_t)k * C + c) * 2 + 0];
     q += partial[((int64_t)k * C + c) * 2 + 1];
   }
-  const double m = (double)N * (double)HW;
-  const double mean_d = s / m;
-  double var = q / m - mean_d * mean_d;
-  if (var < 0.0) var = 0.0;
-  const float mean = (float)mean_d;
-  const float istd = (float)(1.0 / sqrt(var + (double)kEps));
-  if (blockIdx.x < C && threadIdx.x == 0) {  // rows of image 0 publish the statistics
-    save_mean[c] = mean;
-    save_istd[c] = istd;
+  if (BWD) {
+    out0[c] = (float)s;
+    out1[c] = (float)q;
+  } else {
+    const double m = (double)N * (double)HW;
+    const double mean_d = s / m;
+    double var = q / m - mean_d * mean_d;
+    if (var < 0.0) var = 0.0;
+    out0[c] = (float)mean_d;
+    out1[c] = (float)(1.0 / sqrt(var + (double)kEps));
   }
-  const int64_t row = (int64_t)blockIdx.x * HW;
-  for (int i = threadIdx.x; i < HW; i += kThreads) y[row + i] = (x[row + i] - mean) * istd;
 }
 
-__global__ __launch_bounds__(kThreads) void bn_sp_backward_apply_kernel(const float *__restrict__ x,
-                                                                       const float *__restrict__ dy,
-                                                                       float *__restrict__ dx,
-                                                                       const double *__restrict__ partial,
-                                                                       const float *__restrict__ save_mean,
-                                                                       const float *__restrict__ save_istd,
-                                                                       int N, int C, int HW, int chunks) {
-  const int c = blockIdx.x % C;
-  double s1d = 0.0, s2d = 0.0;
-  for (int k = 0; k < chunks; ++k) {
-    s1d += partial[((int64_t)k * C + c) * 2 + 0];
-    s2d += partial[((int64_t)k * C + c) * 2 + 1];
+// Apply pass over the flat tensor, one contiguous run of 1024 units (16 KiB when
+// VEC) per workgroup as in the elementwise engine; a unit (float4 or float) lies
+// inside one (image, channel) row, whose channel is (unit / units per row) % C.
+// FWD: y = (x - mean) * istd.  BWD: dx = istd/m * (m*dy - s1 - xhat*s2).
+template <bool BWD, bool VEC>
+__global__ __launch_bounds__(kThreads) void bn_sp_apply_kernel(const float *__restrict__ x,
+                                                              const float *__restrict__ dy,
+                                                              float *__restrict__ out,
+                                                              const float *__restrict__ p_mean,
+                                                              const float *__restrict__ p_istd,
+                                                              const float *__restrict__ p_s1,
+                                                              const float *__restrict__ p_s2, float m,
+                                                              FastDiv div_row, FastDiv div_c, uint32_t units) {
+  constexpr int W = Unit<VEC>::W;
+  constexpr int kUnroll = 4;
+  const uint32_t base = blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  float xv[kUnroll][W], gv[kUnroll][W] = {};
+  uint32_t ch[kUnroll] = {};
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t unit = base + u * kThreads;
+    if (unit >= units) continue;
+    uint32_t img;
+    div_c.divmod(div_row.div(unit), img, ch[u]);
+    Unit<VEC>::load(x + (int64_t)unit * W, xv[u]);
+    if (BWD) Unit<VEC>::load(dy + (int64_t)unit * W, gv[u]);
   }
-  const float mean = save_mean[c], istd = save_istd[c];
-  const float m = (float)((double)N * (double)HW);
-  const float s1 = (float)s1d, s2 = (float)s2d;
-  const float scale = istd / m;
-  const int64_t row = (int64_t)blockIdx.x * HW;
-  for (int i = threadIdx.x; i < HW; i += kThreads) {
-    const float xh = (x[row + i] - mean) * istd;
-    dx[row + i] = scale * (m * dy[row + i] - s1 - xh * s2);
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t unit = base + u * kThreads;
+    if (unit >= units) continue;
+    const float mean = p_mean[ch[u]], istd = p_istd[ch[u]];
+    float r[W];
+    if (BWD) {
+      const float s1 = p_s1[ch[u]], s2 = p_s2[ch[u]];
+      const float scale = istd / m;
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        const float xh = (xv[u][k] - mean) * istd;
+        r[k] = scale * (m * gv[u][k] - s1 - xh * s2);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < W; ++k) r[k] = (xv[u][k] - mean) * istd;
+    }
+    Unit<VEC>::store(out + (int64_t)unit * W, r);
   }
 }
 
@@ -278,6 +337,8 @@ int check_bn_arrays(const BNDesc *d, const DLArray *a, const DLArray *b) {
   TF_REQUIRE(on_gpu(a) && on_gpu(b), "arrays must live on the GPU");
   const int64_t n = (int64_t)d->N * d->C * d->HW;
   TF_REQUIRE(numel(a) == n && numel(b) == n, "arrays do not match the descriptor");
+  // the spatial kernels index units with 32-bit fast division
+  TF_REQUIRE(d->mode == 0 || n < (int64_t(1) << 31), "spatial mode supports fewer than 2^31 elements");
   return 0;
 }
 
@@ -371,11 +432,22 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
       if (memorytoSaving) *memorytoSaving = shortfall(pbytes);
       return 0;
     }
-    hipLaunchKernelGGL(bn_sp_partial_kernel<false>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x,
-                       (const float *)nullptr, (const float *)nullptr, (const float *)nullptr, partial, d->N,
-                       d->C, d->HW, ipc);
-    hipLaunchKernelGGL(bn_sp_forward_apply_kernel, dim3((unsigned)d->N * d->C), dim3(kThreads), 0, s, x, y,
-                       partial, mean, istd, d->N, d->C, d->HW, real_chunks);
+    const bool vec = d->HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    const int W = vec ? 4 : 1;
+    const FastDiv div_row((uint32_t)(d->HW / W)), div_c((uint32_t)d->C);
+    const uint32_t units = (uint32_t)((int64_t)d->N * d->C * d->HW / W);
+    const dim3 pgrid(d->C, real_chunks), agrid((units + kThreads * 4 - 1) / (kThreads * 4));
+    auto run = [&](auto vec_c) {
+      constexpr bool VEC = decltype(vec_c)::value;
+      hipLaunchKernelGGL((bn_sp_partial_kernel<false, VEC>), pgrid, dim3(kThreads), 0, s, x, (const float *)nullptr,
+                         (const float *)nullptr, (const float *)nullptr, partial, d->N, d->C, d->HW, ipc, div_row);
+      hipLaunchKernelGGL(bn_sp_finish_kernel<false>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, mean,
+                         istd, d->N, d->C, d->HW, real_chunks);
+      hipLaunchKernelGGL((bn_sp_apply_kernel<false, VEC>), agrid, dim3(kThreads), 0, s, x, (const float *)nullptr, y,
+                         (const float *)mean, (const float *)istd, (const float *)nullptr, (const float *)nullptr,
+                         0.f, div_row, div_c, units);
+    };
+    if (vec) run(std::true_type{}); else run(std::false_type{});
     device_free(partial);
   }
   return finish(s, what);
@@ -439,16 +511,32 @@ static int bn_backward_impl(const DLArrayHandle input, const DLArrayHandle doutp
       const int chunks = sp_chunks(d->N, d->C);
       const int ipc = cdiv(d->N, chunks);
       const int real_chunks = cdiv(d->N, ipc);
-      const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double);
+      const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double) + (size_t)d->C * 2 * sizeof(float);
       double *partial = (double *)device_alloc(pbytes);
       if (!partial) {
         if (memorytoSaving) *memorytoSaving = shortfall(pbytes);
         return 0;  // statistics stay published so the call can be repeated
       }
-      hipLaunchKernelGGL(bn_sp_partial_kernel<true>, dim3(d->C, real_chunks), dim3(kThreads), 0, s, x, dy,
-                         mean, istd, partial, d->N, d->C, d->HW, ipc);
-      hipLaunchKernelGGL(bn_sp_backward_apply_kernel, dim3((unsigned)d->N * d->C), dim3(kThreads), 0, s, x,
-                         dy, dx, partial, mean, istd, d->N, d->C, d->HW, real_chunks);
+      // the two per-channel sums of the apply pass live behind the chunk partials
+      float *sums = reinterpret_cast<float *>(partial + (size_t)real_chunks * d->C * 2);
+      const bool vec = d->HW % 4 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) |
+                         reinterpret_cast<uintptr_t>(dx)) & 15u) == 0;
+      const int W = vec ? 4 : 1;
+      const FastDiv div_row((uint32_t)(d->HW / W)), div_c((uint32_t)d->C);
+      const uint32_t units = (uint32_t)((int64_t)d->N * d->C * d->HW / W);
+      const dim3 pgrid(d->C, real_chunks), agrid((units + kThreads * 4 - 1) / (kThreads * 4));
+      const float m = (float)((double)d->N * (double)d->HW);
+      auto run = [&](auto vec_c) {
+        constexpr bool VEC = decltype(vec_c)::value;
+        hipLaunchKernelGGL((bn_sp_partial_kernel<true, VEC>), pgrid, dim3(kThreads), 0, s, x, dy, mean, istd, partial,
+                           d->N, d->C, d->HW, ipc, div_row);
+        hipLaunchKernelGGL(bn_sp_finish_kernel<true>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, sums,
+                           sums + d->C, d->N, d->C, d->HW, real_chunks);
+        hipLaunchKernelGGL((bn_sp_apply_kernel<true, VEC>), agrid, dim3(kThreads), 0, s, x, dy, dx, mean, istd,
+                           (const float *)sums, (const float *)(sums + d->C), m, div_row, div_c, units);
+      };
+      if (vec) run(std::true_type{}); else run(std::false_type{});
       device_free(partial);
     }
   }
