@@ -57,8 +57,54 @@ def _gpu(a, rt):
     return ndarray.array(np.asarray(a, dtype=np.float32), rt.ctx)
 
 
+def _describe(lst, which):
+    """Plan of the launch for `which` (0 forward, 1 grad-data, 2 grad-filter)."""
+    import ctypes
+    from tinyflow_amd import _base
+    buf = ctypes.create_string_buffer(256)
+    assert _base._LIB.DLGpuConvolutionDescribeKernel(lst, which, buf, 256, None) == 0
+    return buf.value.decode()
+
+
 @pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(str(v) for v in c))
 def test_conv_forward_and_gradients(rt, case):
+    _check_conv_case(rt, case)
+
+
+# 3x3 / stride-1 shapes for the Winograd form (forced on: the planner would pick the
+# direct form for most of these small sizes).  (.., expect forward, expect grad-data)
+WINOGRAD_CASES = [
+    ((4, 128, 28, 28, 128, 3, 3, "SAME", 1, 1), True, True),
+    ((4, 512, 7, 7, 512, 3, 3, "SAME", 1, 1), True, True),      # odd extent: half-empty edge tiles
+    ((2, 64, 14, 14, 256, 3, 3, "SAME", 1, 1), True, True),
+    ((3, 8, 5, 5, 12, 3, 3, "SAME", 1, 1), True, True),         # 27 tiles: padded to 28 columns
+    ((1, 4, 7, 9, 4, 3, 3, "SAME", 1, 1), True, True),
+    ((2, 8, 9, 9, 12, 3, 3, "VALID", 1, 1), True, True),        # no padding: grad-data pads by 2
+    ((5, 1, 4, 4, 1, 3, 3, "SAME", 1, 1), False, False),        # one channel: not a multiple of 4
+    ((2, 3, 32, 32, 64, 3, 3, "SAME", 1, 1), False, False),     # 3 input channels
+    ((2, 132, 6, 6, 68, 3, 3, "SAME", 1, 1), True, True),
+    ((2, 8, 8, 8, 6, 3, 3, "SAME", 1, 1), True, False),         # 6 output channels: grad-data reduces over 6
+    ((2, 6, 8, 8, 8, 3, 3, "SAME", 1, 1), False, False),
+    ((130, 4, 2, 2, 4, 3, 3, "SAME", 1, 1), True, True),        # one tile per image
+    ((2, 8, 9, 9, 12, 3, 3, "SAME", 2, 2), False, False),       # strided: never
+]
+
+
+@pytest.mark.parametrize("case,fwd,dgrad", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else str(c))
+def test_conv_winograd_form(rt, monkeypatch, case, fwd, dgrad):
+    from tinyflow_amd import gpu_op
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "1")
+    N, C, H, W, K, R, S, padding, u, v = case
+    _, lst = gpu_op.convolution_2d_forward_get_out_shape((N, C, H, W), (K, C, R, S), "NCHW", padding, u, v)
+    assert ("winograd" in _describe(lst, 0)) == fwd
+    assert ("winograd" in _describe(lst, 1)) == dgrad
+    assert "winograd" not in _describe(lst, 2)
+    _check_conv_case(rt, case)
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "0")
+    assert "winograd" not in _describe(lst, 0) and "winograd" not in _describe(lst, 1)
+
+
+def _check_conv_case(rt, case):
     from tinyflow_amd import gpu_op, ndarray
     N, C, H, W, K, R, S, padding, u, v = case
     rng = np.random.RandomState(abs(hash(case)) % (2 ** 31))

@@ -94,6 +94,21 @@ def test_vgg16_reduced():
 @pytest.mark.parametrize("bn_mode", ["pre_activation", "spatial"])
 def test_resnet_shallow(bn_mode):
     """Five bottlenecks ([2,1,1,1]) at batch 32: well conditioned, plain tolerance."""
+    _resnet_shallow(bn_mode)
+
+
+@pytest.mark.parametrize("config", ["resnet_shallow", "vgg16"])
+def test_train_step_with_winograd_convolutions(monkeypatch, config):
+    """The same steps with every eligible 3x3 convolution and grad-data in the
+    Winograd form (the planner only picks it for larger layers than these)."""
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "1")
+    if config == "vgg16":
+        _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {})
+    else:
+        _resnet_shallow("pre_activation")
+
+
+def _resnet_shallow(bn_mode):
     from tinyflow_amd import models
     from tinyflow_amd.TrainExecute import TrainExecutor
     blocks, batch, lr = [2, 1, 1, 1], 32, 0.01

@@ -320,6 +320,153 @@ __global__ __launch_bounds__(256) void filter_to_krsc_kernel(const float *__rest
   }
 }
 
+// ---- Winograd F(2x2, 3x3) ---------------------------------------------------------
+// A 3x3 / stride-1 correlation evaluated on 2x2 output tiles:
+//   Y = A^T [ (G g G^T) .* (B^T d B) ] A      d: 4x4 input patch, g: 3x3 filter
+// The 16 positions of the transformed domain are independent matrix products
+//   M[pos][mo][t] = sum_cr U[pos][mo][cr] * V[pos][cr][t]     t = (image, tile row, tile column)
+// with 2.25x fewer multiplications than the direct form; they run as one launch of
+// the tile engine with the position on blockIdx.y.  Forward uses it with
+// (mo, cr) = (K, C) on x; grad-data with (mo, cr) = (C, K) on dy and the filter
+// rotated by 180 degrees.  U, V and M live in scratch memory.
+template <class L>
+struct Batched : L {
+  int64_t batch_stride;  // elements between the operands of consecutive problems
+  __device__ inline void init(typename L::State &st, int origin, int tid) const {
+    L one = *this;
+    one.base += (int64_t)blockIdx.y * batch_stride;
+    one.init(st, origin, tid);
+  }
+};
+struct StoreBatched : StoreRowMajor {
+  int64_t batch_stride;
+  template <int TN>
+  __device__ inline void init(State &st, int n0, int lane, int split) const {
+    StoreRowMajor one = *this;
+    one.out += (int64_t)blockIdx.y * batch_stride;
+    one.template init<TN>(st, n0, lane, split);
+  }
+};
+
+// U[pos][k][c] = (G g G^T)[pos], G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1], one lane per
+// filter g = w[k][c] (grad-data: rotated by 180 degrees).  Forward reads U as
+// [mo = k][cr = c], grad-data as its transpose [cr = k][mo = c].
+__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ w, float *__restrict__ U,
+                                                         int K, int C, bool for_dgrad) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= K * C) return;
+  float g[3][3];
+#pragma unroll
+  for (int r = 0; r < 3; ++r)
+#pragma unroll
+    for (int q = 0; q < 3; ++q) g[r][q] = w[(int64_t)idx * 9 + (for_dgrad ? (2 - r) * 3 + (2 - q) : r * 3 + q)];
+  float t[4][3];
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    t[0][q] = g[0][q];
+    t[1][q] = 0.5f * (g[0][q] + g[1][q] + g[2][q]);
+    t[2][q] = 0.5f * (g[0][q] - g[1][q] + g[2][q]);
+    t[3][q] = g[2][q];
+  }
+  const int64_t plane = (int64_t)K * C;
+  const int64_t at = idx;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    U[(i * 4 + 0) * plane + at] = t[i][0];
+    U[(i * 4 + 1) * plane + at] = 0.5f * (t[i][0] + t[i][1] + t[i][2]);
+    U[(i * 4 + 2) * plane + at] = 0.5f * (t[i][0] - t[i][1] + t[i][2]);
+    U[(i * 4 + 3) * plane + at] = t[i][2];
+  }
+}
+
+// V[pos][cr][t] = (B^T d B)[pos], B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]; d is
+// the patch of in[image][cr] whose corner is (2*tile_row - pad_h, 2*tile_col - pad_w),
+// zero outside the image.  One lane per (cr = blockIdx.y, t); columns T..Tp-1 of
+// the padded row are written as zeros.
+__global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
+                                                        int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
+                                                        int pad_w, int T, int Tp) {
+  const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+  const int cr = blockIdx.y;
+  if (t >= (uint32_t)Tp) return;
+  float d[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) d[i][j] = 0.f;
+  if (t < (uint32_t)T) {
+    uint32_t img, rem, th, tw;
+    div_tiles.divmod(t, img, rem);
+    div_tw.divmod(rem, th, tw);
+    const float *plane = in + ((int64_t)img * Cr + cr) * H * W;
+    const int h0 = 2 * (int)th - pad_h, w0 = 2 * (int)tw - pad_w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int h = h0 + i, x = w0 + j;
+        if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = plane[h * W + x];
+      }
+  }
+  float r[4][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    r[0][j] = d[0][j] - d[2][j];
+    r[1][j] = d[1][j] + d[2][j];
+    r[2][j] = d[2][j] - d[1][j];
+    r[3][j] = d[1][j] - d[3][j];
+  }
+  const int64_t plane_sz = (int64_t)Cr * Tp;
+  float *dst = V + (int64_t)cr * Tp + t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    dst[(i * 4 + 0) * plane_sz] = r[i][0] - r[i][2];
+    dst[(i * 4 + 1) * plane_sz] = r[i][1] + r[i][2];
+    dst[(i * 4 + 2) * plane_sz] = r[i][2] - r[i][1];
+    dst[(i * 4 + 3) * plane_sz] = r[i][1] - r[i][3];
+  }
+}
+
+// out[image][mo][2*tile_row + a][2*tile_col + b] = (A^T m A)[a][b], A^T = [1 1 1 0; 0 1 -1 -1],
+// m[pos] = M[pos][mo][t].  One lane per (mo = blockIdx.y, t); `pairs`: Q is even
+// and out 8-byte aligned, so a tile row is one 8-byte store.
+__global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, float *__restrict__ out, int Mo,
+                                                         int P, int Q, FastDiv div_tiles, FastDiv div_tw, int T,
+                                                         int Tp, bool pairs) {
+  const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+  const int mo = blockIdx.y;
+  if (t >= (uint32_t)T) return;
+  const int64_t plane_sz = (int64_t)Mo * Tp;
+  const float *src = M + (int64_t)mo * Tp + t;
+  float m[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m[i][j] = __builtin_nontemporal_load(src + (i * 4 + j) * plane_sz);
+  float s[2][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    s[0][j] = m[0][j] + m[1][j] + m[2][j];
+    s[1][j] = m[1][j] - m[2][j] - m[3][j];
+  }
+  uint32_t img, rem, th, tw;
+  div_tiles.divmod(t, img, rem);
+  div_tw.divmod(rem, th, tw);
+  const int p0 = 2 * (int)th, q0 = 2 * (int)tw;
+  float *dst = out + (((int64_t)img * Mo + mo) * P + p0) * Q + q0;
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    if (p0 + a >= P) break;
+    const float y0 = s[a][0] + s[a][1] + s[a][2], y1 = s[a][1] - s[a][2] - s[a][3];
+    if (pairs) {
+      *reinterpret_cast<float2 *>(dst + a * Q) = make_float2(y0, y1);
+    } else {
+      dst[a * Q] = y0;
+      if (q0 + 1 < Q) dst[a * Q + 1] = y1;
+    }
+  }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 template <int V>
@@ -342,9 +489,9 @@ void with_tile(int bm, int bn, F &&f) {
 thread_local hipEvent_t next_kernel_start = nullptr, next_kernel_stop = nullptr;
 
 template <int BM, int BN, int BK, class AL, class BL, class EP>
-void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s) {
+void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s, int batch = 1) {
   if (next_kernel_start) (void)hipEventRecord(next_kernel_start, s);
-  hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks()), dim3(THREADS), 0, s, al, bl, ep,
+  hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks(), batch), dim3(THREADS), 0, s, al, bl, ep,
                      K, g.k_per_split, g.tiles_m, g.tiles_n);
   if (next_kernel_stop) (void)hipEventRecord(next_kernel_stop, s);
   next_kernel_start = next_kernel_stop = nullptr;
@@ -366,6 +513,7 @@ struct ConvPlan {
   bool a_vec, b_vec;     // operand fetched with the 16-byte loaders (shape permitting)
   int bm, bn, splits;
   int M, N, K;
+  bool winograd = false;  // 3x3 / stride-1 layers: transformed-domain products (bm x bn is their tile)
 };
 
 // Tile and k-split selection.  Every ResNet/VGG layer offers several workable
@@ -382,13 +530,13 @@ struct ConvPlan {
 // It depends on the problem shape and the CU count only, so a given layer always
 // gets the same plan and results stay bit-reproducible from run to run.
 double predict_us(int M, int N, int K, int bm, int bn, int splits, bool wgrad, bool padded, bool scatter,
-                  double out_bytes) {
+                  double out_bytes, int batch = 1) {
   const Geometry g = make_geometry(M, N, K, bm, bn, splits, stage_depth(bm, bn));
   double a = (bm == 128 && bn == 128) ? 0.0705 : (bm == 64 && bn == 128) ? 0.0406 : 0.0229;
   if (padded) a *= 1.04;
   if (wgrad) a *= bm == 128 ? 0.98 : 1.05;
   const double block_us = a * (g.k_per_split + 9.0);
-  const double per_cu = (double)g.blocks() / num_cus();
+  const double per_cu = (double)g.blocks() * batch / num_cus();
   const double whole = std::ceil(per_cu);
   const double rounds = per_cu <= 1.0 ? 1.0 : std::min(whole, per_cu + 0.94);
   const double hiding = whole <= 1 ? 0.656 : whole <= 2 ? 0.84 : whole <= 3 ? 0.92 : 1.0;
@@ -401,7 +549,8 @@ double predict_us(int M, int N, int K, int bm, int bn, int splits, bool wgrad, b
 // Fills p.bm / p.bn / p.splits with the cheapest candidate.  `may_split` is false
 // where the epilogue cannot write partial sums (scatter); grad-filter only has
 // the square tiles.
-void choose_tile_and_splits(ConvPlan &p, bool wgrad, bool padded, bool scatter, bool may_split, double out_bytes) {
+double choose_tile_and_splits(ConvPlan &p, bool wgrad, bool padded, bool scatter, bool may_split,
+                              double out_bytes) {
   static const int tiles[3][2] = {{128, 128}, {64, 128}, {64, 64}};
   const size_t max_scratch = (size_t)512 << 20;
   double best = 1e30;
@@ -436,6 +585,78 @@ void choose_tile_and_splits(ConvPlan &p, bool wgrad, bool padded, bool scatter, 
       }
     }
   }
+  return best;
+}
+
+// Geometry of the Winograd form of a 3x3 / stride-1 convolution (forward) or of its
+// grad-data (the same correlation on dy with padding 2 - pad and the rotated filter).
+struct WinoShape {
+  int Mo, Cr;              // output / reduction channels of the correlation
+  int in_h, in_w, out_h, out_w, pad_h, pad_w;
+  int TH, TW, T, Tp;       // 2x2 output tiles per image column / row, in total, padded to 4
+  size_t u_elems, v_elems, m_elems;  // scratch, each rounded up to 64 floats
+};
+constexpr size_t kMaxWinogradScratch = (size_t)1 << 30;
+
+bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w) {
+  if (d->R != 3 || d->S != 3 || d->u != 1 || d->v != 1 || d->pad_h > 2 || d->pad_w > 2) return false;
+  w.Mo = dgrad ? d->C : d->K;
+  w.Cr = dgrad ? d->K : d->C;
+  w.in_h = dgrad ? d->P : d->H;
+  w.in_w = dgrad ? d->Q : d->W;
+  w.out_h = dgrad ? d->H : d->P;
+  w.out_w = dgrad ? d->W : d->Q;
+  w.pad_h = dgrad ? 2 - d->pad_h : d->pad_h;
+  w.pad_w = dgrad ? 2 - d->pad_w : d->pad_w;
+  // 16-byte loads of U: rows of Cr floats (forward), of Mo floats (grad-data, transposed)
+  if (w.Cr < 4 || w.Cr % 4 != 0 || w.Cr > 65535 || w.Mo < 1 || w.Mo > 65535 || (dgrad && w.Mo % 4 != 0)) return false;
+  w.TH = cdiv(w.out_h, 2);
+  w.TW = cdiv(w.out_w, 2);
+  const int64_t T = (int64_t)d->N * w.TH * w.TW;
+  if (T < 1 || T > (1 << 28)) return false;
+  w.T = (int)T;
+  w.Tp = (w.T + 3) / 4 * 4;
+  auto round64 = [](int64_t n) { return (size_t)((n + 63) / 64 * 64); };
+  w.u_elems = round64((int64_t)16 * w.Mo * w.Cr);
+  w.v_elems = round64((int64_t)16 * w.Cr * w.Tp);
+  w.m_elems = round64((int64_t)16 * w.Mo * w.Tp);
+  if ((w.u_elems + w.v_elems + w.m_elems) * 4 > kMaxWinogradScratch) return false;
+  return true;
+}
+
+// Decides between the direct and the Winograd form and fills the plan of the latter.
+// Model: the 16 transformed-domain products as one batched launch of the tile engine,
+// plus the transform passes at their measured memory rate.  TINYFLOW_WINOGRAD=0 / 1
+// in the environment forces the choice (tests and measurements).
+void consider_winograd(ConvPlan &p, const ConvDesc *d, bool dgrad, double direct_us, const char *variant) {
+  WinoShape w;
+  if (!wino_shape(d, dgrad, w)) return;
+  static const int tiles[3][2] = {{128, 128}, {64, 128}, {64, 64}};
+  double best = 1e30;
+  int bm = 64, bn = 64;
+  for (auto &t : tiles) {
+    if (t[0] == 128 && w.Mo <= 64) continue;
+    const double us = predict_us(w.Mo, w.Tp, w.Cr, t[0], t[1], 1, false, false, false, 0.0, 16);
+    if (us < best) {
+      best = us;
+      bm = t[0];
+      bn = t[1];
+    }
+  }
+  const double in_bytes = 4.0 * d->N * w.Cr * w.in_h * w.in_w, out_bytes = 4.0 * d->N * w.Mo * w.out_h * w.out_w;
+  const double moved = in_bytes + out_bytes + 4.0 * (w.v_elems + w.m_elems) + 8.0 * w.u_elems;
+  const double wino_us = best + moved / 4.0e6 + 6.0;
+  const char *force = getenv("TINYFLOW_WINOGRAD");
+  const bool use = force && *force ? atoi(force) != 0 : wino_us < direct_us;
+  if (!use) return;
+  p.winograd = true;
+  p.variant = variant;
+  p.bm = bm;
+  p.bn = bn;
+  p.splits = 1;
+  p.M = w.Mo;
+  p.N = w.Tp;
+  p.K = w.Cr;
 }
 
 ConvPlan plan_forward(const ConvDesc *d) {
@@ -444,7 +665,7 @@ ConvPlan plan_forward(const ConvDesc *d) {
   p.N = d->N * d->P * d->Q;
   p.K = d->C * d->R * d->S;
   const bool padded = d->pad_h || d->pad_w;
-  choose_tile_and_splits(p, false, padded, false, true, 4.0 * p.M * p.N);
+  const double direct_us = choose_tile_and_splits(p, false, padded, false, true, 4.0 * p.M * p.N);
   p.variant = padded ? "fwd_pad" : "fwd_nopad";
   p.epilogue = "StoreNCHW";
   // filter rows of C*R*S floats; a 1x1 / stride-1 / unpadded input is a plain
@@ -454,6 +675,7 @@ ConvPlan plan_forward(const ConvDesc *d) {
   p.a_loader = p.a_vec ? "Across4" : "PlainAcross";
   p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
   p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
+  consider_winograd(p, d, false, direct_us, "fwd_winograd");
   return p;
 }
 
@@ -467,6 +689,7 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   p.b_mode = 0;
   p.a_vec = d->C % 4 == 0;  // the [(k, r, s)][c] filter has rows of C floats
   p.b_vec = false;
+  double direct_us = -1.0;
   if (RS == 1) {
     p.N = d->N * d->P * d->Q;
     const bool dense = d->u == 1 && d->v == 1;
@@ -479,7 +702,7 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   } else {
     p.N = d->N * d->H * d->W;
     if (d->u == 1 && d->v == 1) {
-      choose_tile_and_splits(p, false, true, false, true, 4.0 * p.M * p.N);
+      direct_us = choose_tile_and_splits(p, false, true, false, true, 4.0 * p.M * p.N);
       p.variant = "dgrad_pad";
       p.b_mode = 1;
     } else {
@@ -492,6 +715,7 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   p.a_loader = p.a_vec ? "Along4" : "PlainAlong";
   p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
   if (p.b_vec) p.b_mode = -1;
+  if (direct_us >= 0.0) consider_winograd(p, d, true, direct_us, "dgrad_winograd");
   return p;
 }
 
@@ -514,6 +738,46 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   return p;
 }
 
+// Runs the planned Winograd form: filter and input transforms, the batched products,
+// the output transform.  Scratch follows the usual convention (shortfall reported
+// through memorytoSaving, nothing written).
+int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in, const float *filter,
+                 float *out, int *memorytoSaving, hipStream_t s) {
+  WinoShape w;
+  if (!wino_shape(d, dgrad, w)) return -1;
+  const size_t bytes = (w.u_elems + w.v_elems + w.m_elems) * sizeof(float);
+  float *U = (float *)device_alloc(bytes);
+  if (!U) {
+    if (memorytoSaving) *memorytoSaving = shortfall(bytes);
+    return 0;
+  }
+  float *V = U + w.u_elems, *Mt = V + w.v_elems;
+  const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
+  hipLaunchKernelGGL(wino_filter_kernel, dim3(cdiv(d->K * d->C, 256)), dim3(256), 0, s, filter, U, d->K, d->C, dgrad);
+  hipLaunchKernelGGL(wino_input_kernel, dim3(cdiv(w.Tp, 256), w.Cr), dim3(256), 0, s, in, V, w.Cr, w.in_h, w.in_w,
+                     div_tiles, div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
+  with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
+    const Geometry g = make_geometry(w.Mo, w.Tp, w.Cr, BM, BN, 1, BK);
+    const uint32_t u_bytes = (uint32_t)((size_t)w.Mo * w.Cr * 4);
+    const Batched<Along4<BN, BK>> bl{{V, (uint32_t)((size_t)w.Cr * w.Tp * 4), w.Tp, w.Tp, w.Cr, FastDiv(ONE_SEGMENT), 0},
+                                     (int64_t)w.Cr * w.Tp};
+    const StoreBatched ep{{Mt, w.Tp, w.Mo, w.Tp, 0}, (int64_t)w.Mo * w.Tp};
+    if (dgrad) {
+      const Batched<Along4<BM, BK>> al{{U, u_bytes, w.Mo, w.Mo, w.Cr, FastDiv(ONE_SEGMENT), 0}, (int64_t)w.Mo * w.Cr};
+      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, 16);
+    } else {
+      const Batched<Across4<BM, BK>> al{{U, u_bytes, w.Cr, w.Mo, w.Cr, FastDiv(ONE_SEGMENT), 0}, (int64_t)w.Mo * w.Cr};
+      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, 16);
+    }
+  });
+  const bool pairs = w.out_w % 2 == 0 && (reinterpret_cast<uintptr_t>(out) & 7u) == 0;
+  hipLaunchKernelGGL(wino_output_kernel, dim3(cdiv(w.T, 256), w.Mo), dim3(256), 0, s, (const float *)Mt, out, w.Mo,
+                     w.out_h, w.out_w, div_tiles, div_tw, w.T, w.Tp, pairs);
+  device_free(U);
+  return 0;
+}
+
 }  // namespace
 
 // Introspection for benchmarks (no counterpart in the reference): describes the
@@ -528,6 +792,19 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
   TF_REQUIRE(which >= 0 && which <= 2 && name && name_len > 0, "bad arguments");
   const ConvPlan p = which == 0 ? plan_forward(d) : which == 1 ? plan_dgrad(d) : plan_wgrad(d);
   const int bk = stage_depth(p.bm, p.bn);
+  if (p.winograd) {
+    // the batched product is the contraction kernel; its flop count is what it
+    // executes (16 products), 2.25x below the direct form's
+    snprintf(name, (size_t)name_len,
+             "%s %dx%d s1 | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<Along4<%d, %d>>, StoreBatched>",
+             p.variant, p.bm, p.bn, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk, p.bn, bk);
+    if (flops) {
+      WinoShape w;
+      wino_shape(d, which == 1, w);
+      *flops = 2.0 * 16.0 * w.Mo * (double)w.Cr * w.T;
+    }
+    return 0;
+  }
   char b_args[32];
   if (p.b_mode >= 0) snprintf(b_args, sizeof b_args, "%d, %d, %d", p.bn, bk, p.b_mode);
   else snprintf(b_args, sizeof b_args, "%d, %d", p.bn, bk);
@@ -607,6 +884,12 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
   const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
   if (K == 0) return DLGpuArraySet(output, 0.f, stream);
+  if (plan.winograd) {
+    if (run_winograd(d, false, plan, (const float *)input->data, (const float *)filter->data, (float *)output->data,
+                     memorytoSaving, s) != 0)
+      return -1;
+    return finish(s, "DLGpuConvolution2DForward");
+  }
   const int bm = plan.bm, bn = plan.bn;
   const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
   float *partial = nullptr;
@@ -672,6 +955,12 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   const int M = plan.M, K = plan.K;
   if (numel(dinput) == 0) return 0;
   if (numel(doutput) == 0) return DLGpuArraySet(dinput, 0.f, stream);
+  if (plan.winograd) {
+    if (run_winograd(d, true, plan, (const float *)doutput->data, (const float *)filter->data, (float *)dinput->data,
+                     memorytoSaving, s) != 0)
+      return -1;
+    return finish(s, "DLGpuConvolutionBackwardData");
+  }
 
   // filter as [(k, r, s)][c]; a 1x1 filter already has that layout
   const float *wt = (const float *)filter->data;
