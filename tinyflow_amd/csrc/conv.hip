@@ -467,6 +467,92 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
   }
 }
 
+// Grad-filter in the same domain: dU[pos][k][c] = sum_t dM[pos][k][t] * V[pos][c][t] with
+// dM = A dY A^T (A = [1 0; 1 1; 1 -1; 0 -1], dY the 2x2 tile of dy, zero beyond the
+// edge) and V the transformed input as in forward; then dw = G^T dU G.
+__global__ __launch_bounds__(256) void wino_dy_kernel(const float *__restrict__ dy, float *__restrict__ dM, int K,
+                                                     int P, int Q, FastDiv div_tiles, FastDiv div_tw, int T, int Tp,
+                                                     bool pairs) {
+  const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+  const int k = blockIdx.y;
+  if (t >= (uint32_t)Tp) return;
+  float y[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  if (t < (uint32_t)T) {
+    uint32_t img, rem, th, tw;
+    div_tiles.divmod(t, img, rem);
+    div_tw.divmod(rem, th, tw);
+    const int p0 = 2 * (int)th, q0 = 2 * (int)tw;
+    const float *src = dy + (((int64_t)img * K + k) * P + p0) * Q + q0;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      if (p0 + a >= P) break;
+      if (pairs) {
+        const float2 v = *reinterpret_cast<const float2 *>(src + a * Q);
+        y[a][0] = v.x;
+        y[a][1] = v.y;
+      } else {
+        y[a][0] = src[a * Q];
+        if (q0 + 1 < Q) y[a][1] = src[a * Q + 1];
+      }
+    }
+  }
+  float r[4][2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    r[0][b] = y[0][b];
+    r[1][b] = y[0][b] + y[1][b];
+    r[2][b] = y[0][b] - y[1][b];
+    r[3][b] = -y[1][b];
+  }
+  const int64_t plane_sz = (int64_t)K * Tp;
+  float *dst = dM + (int64_t)k * Tp + t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    dst[(i * 4 + 0) * plane_sz] = r[i][0];
+    dst[(i * 4 + 1) * plane_sz] = r[i][0] + r[i][1];
+    dst[(i * 4 + 2) * plane_sz] = r[i][0] - r[i][1];
+    dst[(i * 4 + 3) * plane_sz] = -r[i][1];
+  }
+}
+
+// dw[k][c] = G^T (sum over k-splits of dU[split][pos][k][c]) G, G^T = [1 .5 .5 0; 0 .5 -.5 0; 0 .5 .5 1].
+// A workgroup owns 64 filters; lane group g adds the splits of positions 4g..4g+3 in
+// split order (fixed, so the result does not depend on timing), then 64 lanes
+// transform.  KC = K*C.
+__global__ __launch_bounds__(256) void wino_dfilter_kernel(const float *__restrict__ dU, float *__restrict__ dw,
+                                                          int KC, int splits) {
+  __shared__ float u[16][64];
+  const int lane = threadIdx.x & 63, group = threadIdx.x >> 6;
+  const int idx = blockIdx.x * 64 + lane;
+  if (idx < KC) {
+    float acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = dU[(int64_t)(group * 4 + j) * KC + idx];
+    for (int sp = 1; sp < splits; ++sp)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] += dU[((int64_t)sp * 16 + group * 4 + j) * KC + idx];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u[group * 4 + j][lane] = acc[j];
+  }
+  __syncthreads();
+  if (group != 0 || idx >= KC) return;
+  float r[3][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float u0 = u[j][lane], u1 = u[4 + j][lane], u2 = u[8 + j][lane], u3 = u[12 + j][lane];
+    r[0][j] = u0 + 0.5f * (u1 + u2);
+    r[1][j] = 0.5f * (u1 - u2);
+    r[2][j] = 0.5f * (u1 + u2) + u3;
+  }
+  float *dst = dw + (int64_t)idx * 9;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    dst[i * 3 + 0] = r[i][0] + 0.5f * (r[i][1] + r[i][2]);
+    dst[i * 3 + 1] = 0.5f * (r[i][1] - r[i][2]);
+    dst[i * 3 + 2] = 0.5f * (r[i][1] + r[i][2]) + r[i][3];
+  }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 template <int V>
@@ -598,7 +684,7 @@ struct WinoShape {
 };
 constexpr size_t kMaxWinogradScratch = (size_t)1 << 30;
 
-bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w) {
+bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false) {
   if (d->R != 3 || d->S != 3 || d->u != 1 || d->v != 1 || d->pad_h > 2 || d->pad_w > 2) return false;
   w.Mo = dgrad ? d->C : d->K;
   w.Cr = dgrad ? d->K : d->C;
@@ -609,7 +695,9 @@ bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w) {
   w.pad_h = dgrad ? 2 - d->pad_h : d->pad_h;
   w.pad_w = dgrad ? 2 - d->pad_w : d->pad_w;
   // 16-byte loads of U: rows of Cr floats (forward), of Mo floats (grad-data, transposed)
-  if (w.Cr < 4 || w.Cr % 4 != 0 || w.Cr > 65535 || w.Mo < 1 || w.Mo > 65535 || (dgrad && w.Mo % 4 != 0)) return false;
+  // (grad-filter reduces over the tiles instead and has no such condition)
+  if (w.Cr < 1 || w.Cr > 65535 || w.Mo < 1 || w.Mo > 65535) return false;
+  if (!wgrad && (w.Cr % 4 != 0 || (dgrad && w.Mo % 4 != 0))) return false;
   w.TH = cdiv(w.out_h, 2);
   w.TW = cdiv(w.out_w, 2);
   const int64_t T = (int64_t)d->N * w.TH * w.TW;
@@ -617,7 +705,7 @@ bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w) {
   w.T = (int)T;
   w.Tp = (w.T + 3) / 4 * 4;
   auto round64 = [](int64_t n) { return (size_t)((n + 63) / 64 * 64); };
-  w.u_elems = round64((int64_t)16 * w.Mo * w.Cr);
+  w.u_elems = wgrad ? 0 : round64((int64_t)16 * w.Mo * w.Cr);
   w.v_elems = round64((int64_t)16 * w.Cr * w.Tp);
   w.m_elems = round64((int64_t)16 * w.Mo * w.Tp);
   if ((w.u_elems + w.v_elems + w.m_elems) * 4 > kMaxWinogradScratch) return false;
@@ -657,6 +745,46 @@ void consider_winograd(ConvPlan &p, const ConvDesc *d, bool dgrad, double direct
   p.M = w.Mo;
   p.N = w.Tp;
   p.K = w.Cr;
+}
+
+// Grad-filter in the Winograd domain: batched [K x Tp] * [Tp x C] products, split
+// along the tile index where 16 x tiles leave CUs idle.
+void consider_winograd_wgrad(ConvPlan &p, const ConvDesc *d, double direct_us) {
+  WinoShape w;
+  if (!wino_shape(d, false, w, true)) return;
+  static const int tiles[3][2] = {{128, 128}, {64, 128}, {64, 64}};
+  static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+  const double out_bytes = 4.0 * 16.0 * d->K * d->C;
+  double best = 1e30;
+  int bm = 64, bn = 64, best_splits = 1;
+  for (auto &t : tiles) {
+    if (t[0] == 128 && d->K <= 64) continue;
+    if (t[1] == 128 && d->C <= 64) continue;
+    for (int splits : cand) {
+      if (splits > 1 && (w.Tp / splits < 64 || splits * out_bytes > 256e6)) continue;
+      const double us = predict_us(d->K, d->C, w.Tp, t[0], t[1], splits, false, false, false, out_bytes, 16);
+      if (us < best) {
+        best = us;
+        bm = t[0];
+        bn = t[1];
+        best_splits = make_geometry(d->K, d->C, w.Tp, bm, bn, splits, stage_depth(bm, bn)).splits;
+      }
+    }
+  }
+  const double moved = 4.0 * d->N * ((double)d->C * d->H * d->W + (double)d->K * d->P * d->Q) +
+                       4.0 * (w.v_elems + w.m_elems);
+  const double wino_us = best + moved / 4.0e6 + 6.0;
+  const char *force = getenv("TINYFLOW_WINOGRAD");
+  const bool use = force && *force ? atoi(force) != 0 : wino_us < direct_us;
+  if (!use) return;
+  p.winograd = true;
+  p.variant = "wgrad_winograd";
+  p.bm = bm;
+  p.bn = bn;
+  p.splits = best_splits;
+  p.M = d->K;
+  p.N = d->C;
+  p.K = w.Tp;
 }
 
 ConvPlan plan_forward(const ConvDesc *d) {
@@ -725,7 +853,7 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   p.N = d->C * d->R * d->S;
   p.K = d->N * d->P * d->Q;
   const bool padded = d->pad_h || d->pad_w;
-  choose_tile_and_splits(p, true, padded, false, true, 4.0 * p.M * p.N);
+  const double direct_us = choose_tile_and_splits(p, true, padded, false, true, 4.0 * p.M * p.N);
   p.variant = padded ? "wgrad_pad" : "wgrad_nopad";
   p.epilogue = "StoreRowMajor";
   // dy is [image][out channel][pixel]; x is the same kind of block for a 1x1 /
@@ -735,6 +863,7 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   p.a_loader = p.a_vec ? "Across4" : "DyAcross";
   p.b_loader = p.b_vec ? "Across4" : "GatherAcross";
   p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
+  consider_winograd_wgrad(p, d, direct_us);
   return p;
 }
 
@@ -778,6 +907,41 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
   return 0;
 }
 
+int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, const float *dy, float *dw,
+                       int *memorytoSaving, hipStream_t s) {
+  WinoShape w;
+  if (!wino_shape(d, false, w, true)) return -1;
+  const int KC = d->K * d->C;
+  const int bk = stage_depth(plan.bm, plan.bn);
+  const Geometry g = make_geometry(d->K, d->C, w.Tp, plan.bm, plan.bn, plan.splits, bk);
+  const size_t du_elems = (size_t)g.splits * 16 * KC;
+  const size_t bytes = (w.v_elems + w.m_elems + du_elems) * sizeof(float);
+  float *V = (float *)device_alloc(bytes);
+  if (!V) {
+    if (memorytoSaving) *memorytoSaving = shortfall(bytes);
+    return 0;
+  }
+  float *dM = V + w.v_elems, *dU = dM + w.m_elems;
+  const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
+  hipLaunchKernelGGL(wino_input_kernel, dim3(cdiv(w.Tp, 256), d->C), dim3(256), 0, s, x, V, d->C, d->H, d->W,
+                     div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
+  const bool pairs = d->Q % 2 == 0 && (reinterpret_cast<uintptr_t>(dy) & 7u) == 0;
+  hipLaunchKernelGGL(wino_dy_kernel, dim3(cdiv(w.Tp, 256), d->K), dim3(256), 0, s, dy, dM, d->K, d->P, d->Q,
+                     div_tiles, div_tw, w.T, w.Tp, pairs);
+  with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
+    constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
+    const Batched<Across4<BM, BK>> al{{dM, (uint32_t)((size_t)d->K * w.Tp * 4), w.Tp, d->K, w.Tp, FastDiv(ONE_SEGMENT), 0},
+                                      (int64_t)d->K * w.Tp};
+    const Batched<Across4<BN, BK>> bl{{V, (uint32_t)((size_t)d->C * w.Tp * 4), w.Tp, d->C, w.Tp, FastDiv(ONE_SEGMENT), 0},
+                                      (int64_t)d->C * w.Tp};
+    const StoreBatched ep{{dU, d->C, d->K, d->C, (int64_t)16 * KC}, (int64_t)KC};
+    launch<BM, BN, BK>(al, bl, ep, w.Tp, g, s, 16);
+  });
+  hipLaunchKernelGGL(wino_dfilter_kernel, dim3(cdiv(KC, 64)), dim3(256), 0, s, (const float *)dU, dw, KC, g.splits);
+  device_free(V);
+  return 0;
+}
+
 }  // namespace
 
 // Introspection for benchmarks (no counterpart in the reference): describes the
@@ -796,12 +960,13 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
     // the batched product is the contraction kernel; its flop count is what it
     // executes (16 products), 2.25x below the direct form's
     snprintf(name, (size_t)name_len,
-             "%s %dx%d s1 | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<Along4<%d, %d>>, StoreBatched>",
-             p.variant, p.bm, p.bn, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk, p.bn, bk);
+             "%s %dx%d s%d | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<%s<%d, %d>>, StoreBatched>",
+             p.variant, p.bm, p.bn, p.splits, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk,
+             which == 2 ? "Across4" : "Along4", p.bn, bk);
     if (flops) {
       WinoShape w;
-      wino_shape(d, which == 1, w);
-      *flops = 2.0 * 16.0 * w.Mo * (double)w.Cr * w.T;
+      wino_shape(d, which == 1, w, which == 2);
+      *flops = 2.0 * 16.0 * d->K * (double)d->C * w.T;
     }
     return 0;
   }
@@ -1075,6 +1240,12 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
   const int M = plan.M, N = plan.N, K = plan.K;
   if (M == 0 || N == 0) return 0;
   if (K == 0) return DLGpuArraySet(dfilter, 0.f, stream);
+  if (plan.winograd) {
+    if (run_winograd_wgrad(d, plan, (const float *)input->data, (const float *)doutput->data, (float *)dfilter->data,
+                           memorytoSaving, s) != 0)
+      return -1;
+    return finish(s, "DLGpuConvolutionBackwardFilter");
+  }
 
   const int bm = plan.bm, bn = plan.bn;
   Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
