@@ -32,6 +32,11 @@ POOL_CASES = [
     ((2, 3, 9, 10), "max", 1, 1, 1, 2, 3, 3),
     ((2, 3, 9, 10), "max", 2, 2, 2, 1, 5, 4),
     ((16, 64, 112, 112), "max", 1, 1, 2, 2, 3, 3),  # stem pool at full spatial size
+    ((2, 3, 70, 130), "max", 0, 0, 2, 2, 2, 2),     # several tiles per plane, ragged last tile
+    ((2, 3, 33, 67), "max", 1, 1, 2, 2, 3, 3),
+    # windows too large for the one-pass tile kernel: the two-pass kernels
+    ((2, 3, 40, 80), "max", 4, 4, 1, 1, 9, 9),      # stride 1: cell kernel
+    ((2, 3, 40, 90), "max", 0, 0, 3, 3, 15, 15),    # stride 3: per-element kernel
 ]
 
 
@@ -84,8 +89,9 @@ def test_max_pool_routing_is_first_maximum(rt):
     np.testing.assert_array_equal(gdx.asnumpy()[0, 0], expect)
 
 
-@pytest.mark.parametrize("case", [((4, 8, 28, 28), 1, 1, 2, 2, 3, 3), ((2, 3, 11, 13), 0, 0, 3, 3, 3, 3)],
-                         ids=["overlapping", "stride3"])
+@pytest.mark.parametrize("case", [((4, 8, 28, 28), 1, 1, 2, 2, 3, 3), ((2, 3, 40, 80), 4, 4, 1, 1, 9, 9),
+                                  ((2, 3, 40, 90), 0, 0, 3, 3, 15, 15)],
+                         ids=["one-pass", "large-window-stride1", "large-window-stride3"])
 def test_max_pool_backward_without_scratch_memory(rt, case):
     """With no device memory left for the arg-max scratch the backward pass still
     runs (the entry point cannot report out-of-memory) and gives the same bits."""

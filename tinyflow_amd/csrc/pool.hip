@@ -17,6 +17,8 @@
 #include "gemm_core.h"
 #include "internal.h"
 
+#include <algorithm>
+
 using namespace tf;
 using tf::gemm::FastDiv;
 
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void pool_backward_cell_kernel(const unsi
                                                                      const float *__restrict__ dy,
                                                                      float *__restrict__ dx, PoolParams pp,
                                                                      FastDiv div_cells, FastDiv div_cw, int cells_h,
-                                                                     int cells_w, uint32_t total_cells) {
+                                                                     int cells_w, uint32_t total_cells, bool pairs) {
   const uint32_t stride = gridDim.x * kThreads;
   for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < total_cells; i += stride) {
     uint32_t nc, cell, ci, cj;
@@ -180,6 +182,12 @@ __global__ __launch_bounds__(kThreads) void pool_backward_cell_kernel(const unsi
       }
     }
     float *plane = dx + (int64_t)nc * pp.H * pp.W;
+    if (pairs) {  // v == 2, W even, dx 8-byte aligned: a cell row is one 8-byte store
+      *reinterpret_cast<float2 *>(plane + h0 * pp.W + w0) = make_float2(acc[0], acc[1]);
+      if (pp.u == 2 && h0 + 1 < pp.H)
+        *reinterpret_cast<float2 *>(plane + (h0 + 1) * pp.W + w0) = make_float2(acc[2], acc[3]);
+      continue;
+    }
     for (int dh = 0; dh < pp.u; ++dh)
       for (int dw = 0; dw < pp.v; ++dw) {
         const int h = h0 + dh, w = w0 + dw;
@@ -188,6 +196,131 @@ __global__ __launch_bounds__(kThreads) void pool_backward_cell_kernel(const unsi
           plane[h * pp.W + w] = slot == 0 ? acc[0] : slot == 1 ? acc[1] : slot == 2 ? acc[2] : acc[3];
         }
       }
+  }
+}
+
+// Max-pool backward in one pass for the window shapes of the reference models
+// (3x3 and 2x2 at stride 2; template arguments, so every loop below unrolls and
+// every division is by a constant).  A workgroup owns a 16 x 64 tile of dx: it
+// stages the part of x that the tile's windows read in LDS, finds each window's
+// arg-max tap there (same scan as window_argmax, so the same tap), keeps tap and
+// dy per window in LDS, and then every lane gathers four consecutive dx elements
+// from the windows that cover them, in the (p, q) order of the two-pass kernels:
+// same bits, x / dy / dx cross HBM once, and no scratch memory.
+constexpr int kTileH = 16, kTileW = 64;
+
+template <int FH, int FW, int U, int V>
+__global__ __launch_bounds__(kThreads) void pool_max_backward_tile_kernel(const float *__restrict__ x,
+                                                                         const float *__restrict__ dy,
+                                                                         float *__restrict__ dx, PoolParams pp,
+                                                                         FastDiv div_tiles, FastDiv div_tw,
+                                                                         bool vec4) {
+  // windows that can touch the tile, and the rows / columns of x they read
+  constexpr int NP = (kTileH + FH - 2) / U + 2, NQ = (kTileW + FW - 2) / V + 2;
+  constexpr int RH = (NP - 1) * U + FH, RW = (NQ - 1) * V + FW;
+  __shared__ float xs[RH][RW + 1];
+  __shared__ float gs[NP][NQ];
+  __shared__ unsigned char ts[NP][NQ];
+  uint32_t nc, tile, ti, tj;
+  div_tiles.divmod(blockIdx.x, nc, tile);
+  div_tw.divmod(tile, ti, tj);
+  const int h0 = (int)ti * kTileH, w0 = (int)tj * kTileW;
+  // first window row / column that can reach the tile (may lie before window 0)
+  const int p_first = (h0 + pp.pad_h - FH + 1 >= 0) ? (h0 + pp.pad_h - FH + U) / U : 0;
+  const int q_first = (w0 + pp.pad_w - FW + 1 >= 0) ? (w0 + pp.pad_w - FW + V) / V : 0;
+  const int xr0 = p_first * U - pp.pad_h, xc0 = q_first * V - pp.pad_w;  // may be negative
+  const int tid = threadIdx.x;
+  const float *plane = x + (int64_t)nc * pp.H * pp.W;
+  // all loads of a lane are issued before the first one is used
+  constexpr int XPT = (RH * RW + kThreads - 1) / kThreads, WPT = (NP * NQ + kThreads - 1) / kThreads;
+  float xv[XPT];
+#pragma unroll
+  for (int e = 0; e < XPT; ++e) {
+    const int i = tid + e * kThreads;
+    const int r = i / RW, c = i - r * RW;
+    const int h = xr0 + r, w = xc0 + c;
+    xv[e] = (i < RH * RW && (unsigned)h < (unsigned)pp.H && (unsigned)w < (unsigned)pp.W) ? plane[h * pp.W + w] : 0.f;
+  }
+  const float *gplane = dy + (int64_t)nc * pp.P * pp.Q;
+  float gv[WPT];
+#pragma unroll
+  for (int e = 0; e < WPT; ++e) {
+    const int i = tid + e * kThreads;
+    const int pi = i / NQ, qi = i - pi * NQ;
+    const int p = p_first + pi, q = q_first + qi;
+    gv[e] = (i < NP * NQ && p < pp.P && q < pp.Q) ? gplane[p * pp.Q + q] : 0.f;
+  }
+#pragma unroll
+  for (int e = 0; e < XPT; ++e) {
+    const int i = tid + e * kThreads;
+    const int r = i / RW, c = i - r * RW;
+    if (i < RH * RW) xs[r][c] = xv[e];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < WPT; ++e) {
+    const int i = tid + e * kThreads;
+    if (i >= NP * NQ) break;
+    const int pi = i / NQ, qi = i - pi * NQ;
+    const int p = p_first + pi, q = q_first + qi;
+    int arg = 255;
+    const float g = gv[e];
+    if (p < pp.P && q < pp.Q) {
+      float best = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < FH; ++r) {
+        const int h = xr0 + pi * U + r;
+#pragma unroll
+        for (int sft = 0; sft < FW; ++sft) {
+          const int w = xc0 + qi * V + sft;
+          if ((unsigned)h < (unsigned)pp.H && (unsigned)w < (unsigned)pp.W) {
+            const float val = xs[pi * U + r][qi * V + sft];
+            if (val > best || (arg == 255 && val == best)) {
+              best = val;
+              arg = r * FW + sft;
+            }
+          }
+        }
+      }
+    }
+    ts[pi][qi] = (unsigned char)arg;
+    gs[pi][qi] = g;
+  }
+  __syncthreads();
+  const int h = h0 + tid / (kTileW / 4), wq = w0 + (tid % (kTileW / 4)) * 4;
+  if (h >= pp.H || wq >= pp.W) return;
+  float out[4];
+  // windows covering row h: p*U - pad <= h <= p*U - pad + FH - 1
+  const int a_h = h + pp.pad_h - FH + 1;
+  const int pl = a_h <= 0 ? 0 : (a_h + U - 1) / U, ph = (h + pp.pad_h) / U;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int w = wq + k;
+    const int a_w = w + pp.pad_w - FW + 1;
+    const int ql = a_w <= 0 ? 0 : (a_w + V - 1) / V, qh = (w + pp.pad_w) / V;
+    float acc = 0.f;
+#pragma unroll
+    for (int dp = 0; dp < (FH + U - 1) / U; ++dp) {
+      const int p = pl + dp;
+      if (p > ph) break;
+      const int r = h - (p * U - pp.pad_h);
+#pragma unroll
+      for (int dq = 0; dq < (FW + V - 1) / V; ++dq) {
+        const int q = ql + dq;
+        if (q > qh) break;
+        // windows past P / Q hold tap 255 and never match
+        if ((int)ts[p - p_first][q - q_first] == r * FW + (w - (q * V - pp.pad_w))) acc += gs[p - p_first][q - q_first];
+      }
+    }
+    out[k] = acc;
+  }
+  float *dst = dx + (int64_t)nc * pp.H * pp.W + h * pp.W + wq;
+  if (vec4 && wq + 3 < pp.W) {
+    *reinterpret_cast<float4 *>(dst) = make_float4(out[0], out[1], out[2], out[3]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (wq + k < pp.W) dst[k] = out[k];
   }
 }
 
@@ -287,6 +420,22 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
   const PoolParams pp = params_of(d);
   if (d->mode == 0) {
     TF_REQUIRE(d->fh * d->fw < 255, "max-pool windows of 255 or more taps are not supported");
+    const int tiles_h = cdiv(d->H, kTileH), tiles_w = cdiv(d->W, kTileW);
+    const int64_t blocks = (int64_t)d->N * d->C * tiles_h * tiles_w;
+    const bool square2 = d->u == 2 && d->v == 2 && d->fh == d->fw && (d->fh == 2 || d->fh == 3);
+    if (square2 && blocks < ((int64_t)1 << 31)) {
+      const bool vec4 = d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(dinput->data) & 15u) == 0;
+      const FastDiv div_tiles((uint32_t)(tiles_h * tiles_w)), div_tw((uint32_t)tiles_w);
+      const float *xp = (const float *)input->data, *gp = (const float *)doutput->data;
+      float *dp = (float *)dinput->data;
+      if (d->fh == 3)
+        hipLaunchKernelGGL((pool_max_backward_tile_kernel<3, 3, 2, 2>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp,
+                           gp, dp, pp, div_tiles, div_tw, vec4);
+      else
+        hipLaunchKernelGGL((pool_max_backward_tile_kernel<2, 2, 2, 2>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp,
+                           gp, dp, pp, div_tiles, div_tw, vec4);
+      return finish(s, "DLGpuPooling2DBackward");
+    }
     const int64_t windows = numel(doutput);
     // this entry point has no way to report a failed allocation to the caller
     // (no memorytoSaving argument), so it must also work without the scratch
@@ -300,7 +449,8 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
       hipLaunchKernelGGL(pool_backward_cell_kernel, dim3(grid_for(cells)), dim3(kThreads), 0, s, tap,
                          (const float *)doutput->data, (float *)dinput->data, pp,
                          FastDiv((uint32_t)(cells_h * cells_w)), FastDiv((uint32_t)cells_w), cells_h, cells_w,
-                         (uint32_t)cells);
+                         (uint32_t)cells,
+                         pp.v == 2 && pp.W % 2 == 0 && (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0);
     } else {
       hipLaunchKernelGGL(pool_backward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s, tap,
                          (const float *)input->data, (const float *)doutput->data, (float *)dinput->data, pp,
