@@ -75,6 +75,8 @@ def test_conv_forward_and_gradients(rt, case):
 # direct form for most of these small sizes).  (.., expect forward, expect grad-data)
 WINOGRAD_CASES = [
     ((4, 128, 28, 28, 128, 3, 3, "SAME", 1, 1), True, True),
+    ((4, 64, 56, 56, 64, 3, 3, "SAME", 1, 1), True, True),
+    ((2, 64, 30, 26, 128, 3, 3, "SAME", 1, 1), True, True),     # extents that are not multiples of 4
     ((4, 512, 7, 7, 512, 3, 3, "SAME", 1, 1), True, True),      # odd extent: half-empty edge tiles
     ((2, 64, 14, 14, 256, 3, 3, "SAME", 1, 1), True, True),
     ((3, 8, 5, 5, 12, 3, 3, "SAME", 1, 1), True, True),         # 27 tiles: padded to 28 columns
@@ -90,16 +92,19 @@ WINOGRAD_CASES = [
 ]
 
 
+@pytest.mark.parametrize("force", ["2", "4"])
 @pytest.mark.parametrize("case,fwd,dgrad", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else str(c))
-def test_conv_winograd_form(rt, monkeypatch, case, fwd, dgrad):
+def test_conv_winograd_form(rt, monkeypatch, case, fwd, dgrad, force):
+    """F(2x2, 3x3) and F(4x4, 3x3), forced; the latter is limited to 128 reduction channels."""
     from tinyflow_amd import gpu_op
-    monkeypatch.setenv("TINYFLOW_WINOGRAD", "1")
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", force)
     N, C, H, W, K, R, S, padding, u, v = case
     _, lst = gpu_op.convolution_2d_forward_get_out_shape((N, C, H, W), (K, C, R, S), "NCHW", padding, u, v)
-    assert ("winograd" in _describe(lst, 0)) == fwd
-    assert ("winograd" in _describe(lst, 1)) == dgrad
-    # grad-filter reduces over the tiles: no condition on the channel counts
-    assert ("winograd" in _describe(lst, 2)) == (u == 1 and v == 1)
+    tag = "winograd4x4" if force == "4" else "winograd "
+    assert (tag in _describe(lst, 0)) == (fwd and (force == "2" or C <= 128))
+    assert (tag in _describe(lst, 1)) == (dgrad and (force == "2" or K <= 128))
+    # grad-filter reduces over the tiles: no condition on the channel counts; always 2x2 tiles
+    assert ("wgrad_winograd " in _describe(lst, 2)) == (u == 1 and v == 1)
     _check_conv_case(rt, case)
     monkeypatch.setenv("TINYFLOW_WINOGRAD", "0")
     assert not any("winograd" in _describe(lst, which) for which in range(3))

@@ -97,18 +97,22 @@ def test_resnet_shallow(bn_mode):
     _resnet_shallow(bn_mode)
 
 
+@pytest.mark.parametrize("force", ["1", "2", "4"])
 @pytest.mark.parametrize("config", ["resnet_shallow", "vgg16"])
-def test_train_step_with_winograd_convolutions(monkeypatch, config):
-    """The same steps with every eligible 3x3 convolution and grad-data in the
-    Winograd form (the planner only picks it for larger layers than these)."""
-    monkeypatch.setenv("TINYFLOW_WINOGRAD", "1")
+def test_train_step_with_winograd_convolutions(monkeypatch, config, force):
+    """The same steps with every eligible 3x3 convolution, grad-data and grad-filter in a
+    Winograd form: the planner's tile choice (1), F(2x2) or F(4x4) everywhere.  The
+    planner alone only picks them for larger layers than these.  The first step is
+    held to the plain bound; in the second step of the ResNet a single ReLU whose
+    input the different rounding moves across zero shifts a gradient by a few 1e-3."""
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", force)
     if config == "vgg16":
         _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {})
     else:
-        _resnet_shallow("pre_activation")
+        _resnet_shallow("pre_activation", later_steps_bound=1e-2)
 
 
-def _resnet_shallow(bn_mode):
+def _resnet_shallow(bn_mode, later_steps_bound=1e-3):
     from tinyflow_amd import models
     from tinyflow_amd.TrainExecute import TrainExecutor
     blocks, batch, lr = [2, 1, 1, 1], 32, 0.01
@@ -124,10 +128,14 @@ def _resnet_shallow(bn_mode):
         out = ex.run({model.X: X, model.y_: y})
         loss_ref, grads_ref, params, _ = OM.train_step(net, params, X.astype(np.float64), y.astype(np.float64), lr)
         _close(out[0].asnumpy(), loss_ref, "loss step %d" % step, rtol=1e-4)
+        bound = 1e-3 if step == 0 else later_steps_bound
         for var, g in grad_nodes.items():
-            assert _rel_err(ex.value_of(g).asnumpy(), grads_ref[var.name]) <= 1e-3, (step, var.name)
+            assert _rel_err(ex.value_of(g).asnumpy(), grads_ref[var.name]) <= bound, (step, var.name)
         for arr, var in zip(out[1:], model.variables):
-            _close(arr.asnumpy(), params[var.name], "param %s step %d" % (var.name, step))
+            if bound > 1e-3:  # the update carries the gradient's deviation: compare in the same norm
+                assert _rel_err(arr.asnumpy(), params[var.name]) <= bound, (step, var.name)
+            else:
+                _close(arr.asnumpy(), params[var.name], "param %s step %d" % (var.name, step))
 
 
 @pytest.mark.parametrize("bn_mode", ["pre_activation", "spatial"])

@@ -320,12 +320,12 @@ __global__ __launch_bounds__(256) void filter_to_krsc_kernel(const float *__rest
   }
 }
 
-// ---- Winograd F(2x2, 3x3) ---------------------------------------------------------
-// A 3x3 / stride-1 correlation evaluated on 2x2 output tiles:
-//   Y = A^T [ (G g G^T) .* (B^T d B) ] A      d: 4x4 input patch, g: 3x3 filter
-// The 16 positions of the transformed domain are independent matrix products
+// ---- Winograd F(2x2, 3x3) and F(4x4, 3x3) --------------------------------------------
+// A 3x3 / stride-1 correlation evaluated on m x m output tiles (m = 2 or 4):
+//   Y = A^T [ (G g G^T) .* (B^T d B) ] A      d: (m+2) x (m+2) input patch, g: 3x3 filter
+// The (m+2)^2 positions of the transformed domain are independent matrix products
 //   M[pos][mo][t] = sum_cr U[pos][mo][cr] * V[pos][cr][t]     t = (image, tile row, tile column)
-// with 2.25x fewer multiplications than the direct form; they run as one launch of
+// with 2.25x (m = 2) or 4x (m = 4) fewer multiplications than the direct form; they run as one launch of
 // the tile engine with the position on blockIdx.y.  Forward uses it with
 // (mo, cr) = (K, C) on x; grad-data with (mo, cr) = (C, K) on dy and the filter
 // rotated by 180 degrees.  U, V and M live in scratch memory.
@@ -348,121 +348,193 @@ struct StoreBatched : StoreRowMajor {
   }
 };
 
-// U[pos][k][c] = (G g G^T)[pos], G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1], one lane per
-// filter g = w[k][c] (grad-data: rotated by 180 degrees).  Forward reads U as
-// [mo = k][cr = c], grad-data as its transpose [cr = k][mo = c].
+// The 1-D transforms of F(m x m, 3 x 3) for output tiles of m = 2 and m = 4 (patches of
+// 4 and 6); every 2-D transform below applies one of them to the columns and then to
+// the rows.  F(4x4) needs 4x instead of 2.25x fewer multiplications and moves 2.25x
+// instead of 4x the input through the transformed domain, but its larger
+// coefficients cost about one decimal digit; the planner only uses it for forward
+// and grad-data with at most 128 reduction channels.
+template <int TILE>
+struct Wino;
+template <>
+struct Wino<2> {
+  static constexpr int A = 4;
+  // B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
+  __device__ static inline void bt(const float (&d)[4], float (&t)[4]) {
+    t[0] = d[0] - d[2];
+    t[1] = d[1] + d[2];
+    t[2] = d[2] - d[1];
+    t[3] = d[1] - d[3];
+  }
+  // G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]
+  __device__ static inline void g(const float (&f)[3], float (&u)[4]) {
+    u[0] = f[0];
+    u[1] = 0.5f * (f[0] + f[1] + f[2]);
+    u[2] = 0.5f * (f[0] - f[1] + f[2]);
+    u[3] = f[2];
+  }
+  // A^T = [1 1 1 0; 0 1 -1 -1]
+  __device__ static inline void at(const float (&m)[4], float (&y)[2]) {
+    y[0] = m[0] + m[1] + m[2];
+    y[1] = m[1] - m[2] - m[3];
+  }
+};
+template <>
+struct Wino<4> {
+  static constexpr int A = 6;
+  // B^T = [4 0 -5 0 1 0; 0 -4 -4 1 1 0; 0 4 -4 -1 1 0; 0 -2 -1 2 1 0; 0 2 -1 -2 1 0; 0 4 0 -5 0 1]
+  __device__ static inline void bt(const float (&d)[6], float (&t)[6]) {
+    t[0] = 4.f * d[0] - 5.f * d[2] + d[4];
+    t[1] = (d[3] + d[4]) - 4.f * (d[1] + d[2]);
+    t[2] = 4.f * (d[1] - d[2]) + (d[4] - d[3]);
+    t[3] = 2.f * (d[3] - d[1]) + (d[4] - d[2]);
+    t[4] = 2.f * (d[1] - d[3]) + (d[4] - d[2]);
+    t[5] = 4.f * d[1] - 5.f * d[3] + d[5];
+  }
+  // G = [1/4 0 0; -1/6 -1/6 -1/6; -1/6 1/6 -1/6; 1/24 1/12 1/6; 1/24 -1/12 1/6; 0 0 1]
+  __device__ static inline void g(const float (&f)[3], float (&u)[6]) {
+    u[0] = 0.25f * f[0];
+    u[1] = (-1.f / 6.f) * (f[0] + f[1] + f[2]);
+    u[2] = (-1.f / 6.f) * (f[0] - f[1] + f[2]);
+    u[3] = (1.f / 24.f) * f[0] + (1.f / 12.f) * f[1] + (1.f / 6.f) * f[2];
+    u[4] = (1.f / 24.f) * f[0] - (1.f / 12.f) * f[1] + (1.f / 6.f) * f[2];
+    u[5] = f[2];
+  }
+  // A^T = [1 1 1 1 1 0; 0 1 -1 2 -2 0; 0 1 1 4 4 0; 0 1 -1 8 -8 1]
+  __device__ static inline void at(const float (&m)[6], float (&y)[4]) {
+    const float a = m[1] + m[2], b = m[1] - m[2], c = m[3] + m[4], e = m[3] - m[4];
+    y[0] = m[0] + a + c;
+    y[1] = b + 2.f * e;
+    y[2] = a + 4.f * c;
+    y[3] = b + 8.f * e + m[5];
+  }
+};
+
+// U[pos][k][c] = (G g G^T)[pos], one lane per filter g = w[k][c] (grad-data: rotated by
+// 180 degrees).  Forward reads U as [mo = k][cr = c], grad-data as its transpose
+// [cr = k][mo = c].
+template <int TILE>
 __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ w, float *__restrict__ U,
                                                          int K, int C, bool for_dgrad) {
+  constexpr int A = Wino<TILE>::A;
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= K * C) return;
-  float g[3][3];
-#pragma unroll
-  for (int r = 0; r < 3; ++r)
-#pragma unroll
-    for (int q = 0; q < 3; ++q) g[r][q] = w[(int64_t)idx * 9 + (for_dgrad ? (2 - r) * 3 + (2 - q) : r * 3 + q)];
-  float t[4][3];
+  float t[A][3];  // G g, column by column
 #pragma unroll
   for (int q = 0; q < 3; ++q) {
-    t[0][q] = g[0][q];
-    t[1][q] = 0.5f * (g[0][q] + g[1][q] + g[2][q]);
-    t[2][q] = 0.5f * (g[0][q] - g[1][q] + g[2][q]);
-    t[3][q] = g[2][q];
+    float col[3], u[A];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) col[r] = w[(int64_t)idx * 9 + (for_dgrad ? (2 - r) * 3 + (2 - q) : r * 3 + q)];
+    Wino<TILE>::g(col, u);
+#pragma unroll
+    for (int i = 0; i < A; ++i) t[i][q] = u[i];
   }
   const int64_t plane = (int64_t)K * C;
-  const int64_t at = idx;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    U[(i * 4 + 0) * plane + at] = t[i][0];
-    U[(i * 4 + 1) * plane + at] = 0.5f * (t[i][0] + t[i][1] + t[i][2]);
-    U[(i * 4 + 2) * plane + at] = 0.5f * (t[i][0] - t[i][1] + t[i][2]);
-    U[(i * 4 + 3) * plane + at] = t[i][2];
+  for (int i = 0; i < A; ++i) {
+    float u[A];
+    Wino<TILE>::g(t[i], u);
+#pragma unroll
+    for (int j = 0; j < A; ++j) U[(i * A + j) * plane + idx] = u[j];
   }
 }
 
-// V[pos][cr][t] = (B^T d B)[pos], B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]; d is
-// the patch of in[image][cr] whose corner is (2*tile_row - pad_h, 2*tile_col - pad_w),
-// zero outside the image.  One lane per (cr = blockIdx.y, t); columns T..Tp-1 of
-// the padded row are written as zeros.
+// V[pos][cr][t] = (B^T d B)[pos]; d is the patch of in[image][cr] whose corner is
+// (TILE*tile_row - pad_h, TILE*tile_col - pad_w), zero outside the image.  One lane per
+// (cr = blockIdx.y, t); columns T..Tp-1 of the padded row are written as zeros.
+template <int TILE>
 __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
                                                         int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
                                                         int pad_w, int T, int Tp) {
+  constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int cr = blockIdx.y;
   if (t >= (uint32_t)Tp) return;
-  float d[4][4];
+  float d[A][A];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < A; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) d[i][j] = 0.f;
+    for (int j = 0; j < A; ++j) d[i][j] = 0.f;
   if (t < (uint32_t)T) {
     uint32_t img, rem, th, tw;
     div_tiles.divmod(t, img, rem);
     div_tw.divmod(rem, th, tw);
     const float *plane = in + ((int64_t)img * Cr + cr) * H * W;
-    const int h0 = 2 * (int)th - pad_h, w0 = 2 * (int)tw - pad_w;
+    const int h0 = TILE * (int)th - pad_h, w0 = TILE * (int)tw - pad_w;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < A; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < A; ++j) {
         const int h = h0 + i, x = w0 + j;
         if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = plane[h * W + x];
       }
   }
-  float r[4][4];
+  float r[A][A];  // B^T d, column by column
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    r[0][j] = d[0][j] - d[2][j];
-    r[1][j] = d[1][j] + d[2][j];
-    r[2][j] = d[2][j] - d[1][j];
-    r[3][j] = d[1][j] - d[3][j];
+  for (int j = 0; j < A; ++j) {
+    float col[A], o[A];
+#pragma unroll
+    for (int i = 0; i < A; ++i) col[i] = d[i][j];
+    Wino<TILE>::bt(col, o);
+#pragma unroll
+    for (int i = 0; i < A; ++i) r[i][j] = o[i];
   }
   const int64_t plane_sz = (int64_t)Cr * Tp;
   float *dst = V + (int64_t)cr * Tp + t;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    dst[(i * 4 + 0) * plane_sz] = r[i][0] - r[i][2];
-    dst[(i * 4 + 1) * plane_sz] = r[i][1] + r[i][2];
-    dst[(i * 4 + 2) * plane_sz] = r[i][2] - r[i][1];
-    dst[(i * 4 + 3) * plane_sz] = r[i][1] - r[i][3];
+  for (int i = 0; i < A; ++i) {
+    float o[A];
+    Wino<TILE>::bt(r[i], o);
+#pragma unroll
+    for (int j = 0; j < A; ++j) dst[(i * A + j) * plane_sz] = o[j];
   }
 }
 
-// out[image][mo][2*tile_row + a][2*tile_col + b] = (A^T m A)[a][b], A^T = [1 1 1 0; 0 1 -1 -1],
-// m[pos] = M[pos][mo][t].  One lane per (mo = blockIdx.y, t); `pairs`: Q is even
-// and out 8-byte aligned, so a tile row is one 8-byte store.
+// out[image][mo][TILE*tile_row + a][TILE*tile_col + b] = (A^T m A)[a][b], m[pos] = M[pos][mo][t].
+// One lane per (mo = blockIdx.y, t); `rows_vec`: Q is a multiple of TILE and out is
+// aligned to a tile row, which is then one 8- or 16-byte store.
+template <int TILE>
 __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, float *__restrict__ out, int Mo,
                                                          int P, int Q, FastDiv div_tiles, FastDiv div_tw, int T,
-                                                         int Tp, bool pairs) {
+                                                         int Tp, bool rows_vec) {
+  constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int mo = blockIdx.y;
   if (t >= (uint32_t)T) return;
   const int64_t plane_sz = (int64_t)Mo * Tp;
   const float *src = M + (int64_t)mo * Tp + t;
-  float m[4][4];
+  float m[A][A];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < A; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) m[i][j] = __builtin_nontemporal_load(src + (i * 4 + j) * plane_sz);
-  float s[2][4];
+    for (int j = 0; j < A; ++j) m[i][j] = __builtin_nontemporal_load(src + (i * A + j) * plane_sz);
+  float s[TILE][A];  // A^T m, column by column
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    s[0][j] = m[0][j] + m[1][j] + m[2][j];
-    s[1][j] = m[1][j] - m[2][j] - m[3][j];
+  for (int j = 0; j < A; ++j) {
+    float col[A], o[TILE];
+#pragma unroll
+    for (int i = 0; i < A; ++i) col[i] = m[i][j];
+    Wino<TILE>::at(col, o);
+#pragma unroll
+    for (int a = 0; a < TILE; ++a) s[a][j] = o[a];
   }
   uint32_t img, rem, th, tw;
   div_tiles.divmod(t, img, rem);
   div_tw.divmod(rem, th, tw);
-  const int p0 = 2 * (int)th, q0 = 2 * (int)tw;
+  const int p0 = TILE * (int)th, q0 = TILE * (int)tw;
   float *dst = out + (((int64_t)img * Mo + mo) * P + p0) * Q + q0;
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
+  for (int a = 0; a < TILE; ++a) {
     if (p0 + a >= P) break;
-    const float y0 = s[a][0] + s[a][1] + s[a][2], y1 = s[a][1] - s[a][2] - s[a][3];
-    if (pairs) {
-      *reinterpret_cast<float2 *>(dst + a * Q) = make_float2(y0, y1);
+    float y[TILE];
+    Wino<TILE>::at(s[a], y);
+    if (rows_vec) {
+      if constexpr (TILE == 2) *reinterpret_cast<float2 *>(dst + a * Q) = make_float2(y[0], y[1]);
+      else *reinterpret_cast<float4 *>(dst + a * Q) = make_float4(y[0], y[1], y[2], y[3]);
     } else {
-      dst[a * Q] = y0;
-      if (q0 + 1 < Q) dst[a * Q + 1] = y1;
+#pragma unroll
+      for (int b2 = 0; b2 < TILE; ++b2)
+        if (q0 + b2 < Q) dst[a * Q + b2] = y[b2];
     }
   }
 }
@@ -600,6 +672,7 @@ struct ConvPlan {
   int bm, bn, splits;
   int M, N, K;
   bool winograd = false;  // 3x3 / stride-1 layers: transformed-domain products (bm x bn is their tile)
+  int wino_tile = 2;      // F(2x2, 3x3) or F(4x4, 3x3)
 };
 
 // Tile and k-split selection.  Every ResNet/VGG layer offers several workable
@@ -679,12 +752,17 @@ double choose_tile_and_splits(ConvPlan &p, bool wgrad, bool padded, bool scatter
 struct WinoShape {
   int Mo, Cr;              // output / reduction channels of the correlation
   int in_h, in_w, out_h, out_w, pad_h, pad_w;
-  int TH, TW, T, Tp;       // 2x2 output tiles per image column / row, in total, padded to 4
+  int tile, positions;     // output tile edge m (2 or 4) and (m + 2)^2
+  int TH, TW, T, Tp;       // output tiles per image column / row, in total, padded to 4
   size_t u_elems, v_elems, m_elems;  // scratch, each rounded up to 64 floats
 };
+constexpr int kMaxChannelsF4 = 128;  // F(4x4) only up to this many reduction channels (accuracy)
 constexpr size_t kMaxWinogradScratch = (size_t)1 << 30;
 
-bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false) {
+bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false, int tile = 2) {
+  if (tile != 2 && (tile != 4 || wgrad)) return false;
+  w.tile = tile;
+  w.positions = (tile + 2) * (tile + 2);
   if (d->R != 3 || d->S != 3 || d->u != 1 || d->v != 1 || d->pad_h > 2 || d->pad_w > 2) return false;
   w.Mo = dgrad ? d->C : d->K;
   w.Cr = dgrad ? d->K : d->C;
@@ -698,53 +776,77 @@ bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false)
   // (grad-filter reduces over the tiles instead and has no such condition)
   if (w.Cr < 1 || w.Cr > 65535 || w.Mo < 1 || w.Mo > 65535) return false;
   if (!wgrad && (w.Cr % 4 != 0 || (dgrad && w.Mo % 4 != 0))) return false;
-  w.TH = cdiv(w.out_h, 2);
-  w.TW = cdiv(w.out_w, 2);
+  if (tile == 4 && w.Cr > kMaxChannelsF4) return false;
+  w.TH = cdiv(w.out_h, tile);
+  w.TW = cdiv(w.out_w, tile);
   const int64_t T = (int64_t)d->N * w.TH * w.TW;
   if (T < 1 || T > (1 << 28)) return false;
   w.T = (int)T;
   w.Tp = (w.T + 3) / 4 * 4;
   auto round64 = [](int64_t n) { return (size_t)((n + 63) / 64 * 64); };
-  w.u_elems = wgrad ? 0 : round64((int64_t)16 * w.Mo * w.Cr);
-  w.v_elems = round64((int64_t)16 * w.Cr * w.Tp);
-  w.m_elems = round64((int64_t)16 * w.Mo * w.Tp);
+  w.u_elems = wgrad ? 0 : round64((int64_t)w.positions * w.Mo * w.Cr);
+  w.v_elems = round64((int64_t)w.positions * w.Cr * w.Tp);
+  w.m_elems = round64((int64_t)w.positions * w.Mo * w.Tp);
   if ((w.u_elems + w.v_elems + w.m_elems) * 4 > kMaxWinogradScratch) return false;
   return true;
 }
 
-// Decides between the direct and the Winograd form and fills the plan of the latter.
-// Model: the 16 transformed-domain products as one batched launch of the tile engine,
-// plus the transform passes at their measured memory rate.  TINYFLOW_WINOGRAD=0 / 1
-// in the environment forces the choice (tests and measurements).
-void consider_winograd(ConvPlan &p, const ConvDesc *d, bool dgrad, double direct_us, const char *variant) {
-  WinoShape w;
-  if (!wino_shape(d, dgrad, w)) return;
+// Decides between the direct and the Winograd forms and fills the plan of the latter.
+// Model: the transformed-domain products as one batched launch of the tile engine,
+// plus the transform passes at their measured memory rate.  TINYFLOW_WINOGRAD in the
+// environment forces the choice (tests and measurements): 0 direct, 1 Winograd with
+// the model's tile, 2 / 4 that tile where the shape allows it; TINYFLOW_WINOGRAD_MAX_TILE=2
+// keeps the planner to F(2x2) for callers who want its rounding error (that of the
+// direct form) rather than F(4x4)'s (about ten times that).
+void consider_winograd(ConvPlan &p, const ConvDesc *d, bool dgrad, double direct_us, const char *variant2,
+                       const char *variant4) {
+  const char *force = getenv("TINYFLOW_WINOGRAD");
+  const int forced = force && *force ? atoi(force) : -1;
+  if (forced == 0) return;
   static const int tiles[3][2] = {{128, 128}, {64, 128}, {64, 64}};
-  double best = 1e30;
-  int bm = 64, bn = 64;
-  for (auto &t : tiles) {
-    if (t[0] == 128 && w.Mo <= 64) continue;
-    const double us = predict_us(w.Mo, w.Tp, w.Cr, t[0], t[1], 1, false, false, false, 0.0, 16);
-    if (us < best) {
-      best = us;
-      bm = t[0];
-      bn = t[1];
+  double best_us = 1e30;
+  int best_tile = 0, best_bm = 64, best_bn = 64;
+  WinoShape best_w;
+  const char *cap = getenv("TINYFLOW_WINOGRAD_MAX_TILE");
+  const int max_tile = cap && *cap ? atoi(cap) : 4;
+  for (int tile : {2, 4}) {
+    if ((forced == 2 || forced == 4) ? tile != forced : tile > max_tile) continue;
+    WinoShape w;
+    if (!wino_shape(d, dgrad, w, false, tile)) continue;
+    double best = 1e30;
+    int bm = 64, bn = 64;
+    for (auto &t : tiles) {
+      if (t[0] == 128 && w.Mo <= 64) continue;
+      const double us = predict_us(w.Mo, w.Tp, w.Cr, t[0], t[1], 1, false, false, false, 0.0, w.positions);
+      if (us < best) {
+        best = us;
+        bm = t[0];
+        bn = t[1];
+      }
+    }
+    const double in_bytes = 4.0 * d->N * w.Cr * w.in_h * w.in_w, out_bytes = 4.0 * d->N * w.Mo * w.out_h * w.out_w;
+    const double moved = in_bytes + out_bytes + 4.0 * (w.v_elems + w.m_elems) + 8.0 * w.u_elems;
+    // short reductions: the products themselves stream V and M once more
+    const double stream_us = 4.0 * (w.v_elems + w.m_elems) / 5.0e6;
+    const double wino_us = std::max(best, stream_us) + moved / 4.0e6 + 6.0;
+    if (wino_us < best_us) {
+      best_us = wino_us;
+      best_tile = tile;
+      best_bm = bm;
+      best_bn = bn;
+      best_w = w;
     }
   }
-  const double in_bytes = 4.0 * d->N * w.Cr * w.in_h * w.in_w, out_bytes = 4.0 * d->N * w.Mo * w.out_h * w.out_w;
-  const double moved = in_bytes + out_bytes + 4.0 * (w.v_elems + w.m_elems) + 8.0 * w.u_elems;
-  const double wino_us = best + moved / 4.0e6 + 6.0;
-  const char *force = getenv("TINYFLOW_WINOGRAD");
-  const bool use = force && *force ? atoi(force) != 0 : wino_us < direct_us;
-  if (!use) return;
+  if (best_tile == 0 || (forced < 0 && best_us >= direct_us)) return;
   p.winograd = true;
-  p.variant = variant;
-  p.bm = bm;
-  p.bn = bn;
+  p.wino_tile = best_tile;
+  p.variant = best_tile == 2 ? variant2 : variant4;
+  p.bm = best_bm;
+  p.bn = best_bn;
   p.splits = 1;
-  p.M = w.Mo;
-  p.N = w.Tp;
-  p.K = w.Cr;
+  p.M = best_w.Mo;
+  p.N = best_w.Tp;
+  p.K = best_w.Cr;
 }
 
 // Grad-filter in the Winograd domain: batched [K x Tp] * [Tp x C] products, split
@@ -778,6 +880,7 @@ void consider_winograd_wgrad(ConvPlan &p, const ConvDesc *d, double direct_us) {
   const bool use = force && *force ? atoi(force) != 0 : wino_us < direct_us;
   if (!use) return;
   p.winograd = true;
+  p.wino_tile = 2;
   p.variant = "wgrad_winograd";
   p.bm = bm;
   p.bn = bn;
@@ -803,7 +906,7 @@ ConvPlan plan_forward(const ConvDesc *d) {
   p.a_loader = p.a_vec ? "Across4" : "PlainAcross";
   p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
   p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
-  consider_winograd(p, d, false, direct_us, "fwd_winograd");
+  consider_winograd(p, d, false, direct_us, "fwd_winograd", "fwd_winograd4x4");
   return p;
 }
 
@@ -843,7 +946,7 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   p.a_loader = p.a_vec ? "Along4" : "PlainAlong";
   p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
   if (p.b_vec) p.b_mode = -1;
-  if (direct_us >= 0.0) consider_winograd(p, d, true, direct_us, "dgrad_winograd");
+  if (direct_us >= 0.0) consider_winograd(p, d, true, direct_us, "dgrad_winograd", "dgrad_winograd4x4");
   return p;
 }
 
@@ -873,7 +976,7 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
 int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in, const float *filter,
                  float *out, int *memorytoSaving, hipStream_t s) {
   WinoShape w;
-  if (!wino_shape(d, dgrad, w)) return -1;
+  if (!wino_shape(d, dgrad, w, false, plan.wino_tile)) return -1;
   const size_t bytes = (w.u_elems + w.v_elems + w.m_elems) * sizeof(float);
   float *U = (float *)device_alloc(bytes);
   if (!U) {
@@ -882,9 +985,14 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
   }
   float *V = U + w.u_elems, *Mt = V + w.v_elems;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
-  hipLaunchKernelGGL(wino_filter_kernel, dim3(cdiv(d->K * d->C, 256)), dim3(256), 0, s, filter, U, d->K, d->C, dgrad);
-  hipLaunchKernelGGL(wino_input_kernel, dim3(cdiv(w.Tp, 256), w.Cr), dim3(256), 0, s, in, V, w.Cr, w.in_h, w.in_w,
-                     div_tiles, div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
+  const dim3 fgrid(cdiv(d->K * d->C, 256)), igrid(cdiv(w.Tp, 256), w.Cr), ogrid(cdiv(w.T, 256), w.Mo), block(256);
+  auto transforms_in = [&](auto tile_c) {
+    constexpr int TILE = decltype(tile_c)::value;
+    hipLaunchKernelGGL(wino_filter_kernel<TILE>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad);
+    hipLaunchKernelGGL(wino_input_kernel<TILE>, igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles, div_tw,
+                       w.pad_h, w.pad_w, w.T, w.Tp);
+  };
+  if (w.tile == 2) transforms_in(IC<2>{}); else transforms_in(IC<4>{});
   with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     const Geometry g = make_geometry(w.Mo, w.Tp, w.Cr, BM, BN, 1, BK);
@@ -894,15 +1002,19 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
     const StoreBatched ep{{Mt, w.Tp, w.Mo, w.Tp, 0}, (int64_t)w.Mo * w.Tp};
     if (dgrad) {
       const Batched<Along4<BM, BK>> al{{U, u_bytes, w.Mo, w.Mo, w.Cr, FastDiv(ONE_SEGMENT), 0}, (int64_t)w.Mo * w.Cr};
-      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, 16);
+      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, w.positions);
     } else {
       const Batched<Across4<BM, BK>> al{{U, u_bytes, w.Cr, w.Mo, w.Cr, FastDiv(ONE_SEGMENT), 0}, (int64_t)w.Mo * w.Cr};
-      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, 16);
+      launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, w.positions);
     }
   });
-  const bool pairs = w.out_w % 2 == 0 && (reinterpret_cast<uintptr_t>(out) & 7u) == 0;
-  hipLaunchKernelGGL(wino_output_kernel, dim3(cdiv(w.T, 256), w.Mo), dim3(256), 0, s, (const float *)Mt, out, w.Mo,
-                     w.out_h, w.out_w, div_tiles, div_tw, w.T, w.Tp, pairs);
+  const bool rows_vec = w.out_w % w.tile == 0 && (reinterpret_cast<uintptr_t>(out) & (uintptr_t)(4 * w.tile - 1)) == 0;
+  if (w.tile == 2)
+    hipLaunchKernelGGL(wino_output_kernel<2>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
+                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
+  else
+    hipLaunchKernelGGL(wino_output_kernel<4>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
+                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
   device_free(U);
   return 0;
 }
@@ -923,7 +1035,7 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
   }
   float *dM = V + w.v_elems, *dU = dM + w.m_elems;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
-  hipLaunchKernelGGL(wino_input_kernel, dim3(cdiv(w.Tp, 256), d->C), dim3(256), 0, s, x, V, d->C, d->H, d->W,
+  hipLaunchKernelGGL(wino_input_kernel<2>, dim3(cdiv(w.Tp, 256), d->C), dim3(256), 0, s, x, V, d->C, d->H, d->W,
                      div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
   const bool pairs = d->Q % 2 == 0 && (reinterpret_cast<uintptr_t>(dy) & 7u) == 0;
   hipLaunchKernelGGL(wino_dy_kernel, dim3(cdiv(w.Tp, 256), d->K), dim3(256), 0, s, dy, dM, d->K, d->P, d->Q,
@@ -958,15 +1070,15 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
   const int bk = stage_depth(p.bm, p.bn);
   if (p.winograd) {
     // the batched product is the contraction kernel; its flop count is what it
-    // executes (16 products), 2.25x below the direct form's
+    // executes (16 or 36 products), 2.25x or 4x below the direct form's
     snprintf(name, (size_t)name_len,
              "%s %dx%d s%d | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<%s<%d, %d>>, StoreBatched>",
              p.variant, p.bm, p.bn, p.splits, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk,
              which == 2 ? "Across4" : "Along4", p.bn, bk);
     if (flops) {
       WinoShape w;
-      wino_shape(d, which == 1, w, which == 2);
-      *flops = 2.0 * 16.0 * d->K * (double)d->C * w.T;
+      wino_shape(d, which == 1, w, which == 2, p.wino_tile);
+      *flops = 2.0 * w.positions * d->K * (double)d->C * w.T;
     }
     return 0;
   }
