@@ -757,7 +757,7 @@ struct WinoShape {
   size_t u_elems, v_elems, m_elems;  // scratch, each rounded up to 64 floats
 };
 constexpr int kMaxChannelsF4 = 128;  // F(4x4) only up to this many reduction channels (accuracy)
-constexpr size_t kMaxWinogradScratch = (size_t)1 << 30;
+constexpr size_t kMaxWinogradScratch = (size_t)2 << 30;
 
 bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false, int tile = 2) {
   if (tile != 2 && (tile != 4 || wgrad)) return false;
