@@ -103,8 +103,10 @@ def test_conv_winograd_form(rt, monkeypatch, case, fwd, dgrad, force):
     tag = "winograd4x4" if force == "4" else "winograd "
     assert (tag in _describe(lst, 0)) == (fwd and (force == "2" or C <= 128))
     assert (tag in _describe(lst, 1)) == (dgrad and (force == "2" or K <= 128))
-    # grad-filter reduces over the tiles: no condition on the channel counts; always 2x2 tiles
-    assert ("wgrad_winograd " in _describe(lst, 2)) == (u == 1 and v == 1)
+    # grad-filter reduces over the tiles: no condition on the channel counts for 2x2 tiles,
+    # which also stand in where 4x4 tiles are not allowed (more than 128 channels)
+    wtag = "wgrad_winograd4x4" if force == "4" and C <= 128 and K <= 128 else "wgrad_winograd "
+    assert (wtag in _describe(lst, 2)) == (u == 1 and v == 1)
     _check_conv_case(rt, case)
     monkeypatch.setenv("TINYFLOW_WINOGRAD", "0")
     assert not any("winograd" in _describe(lst, which) for which in range(3))

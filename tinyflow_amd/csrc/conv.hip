@@ -378,6 +378,18 @@ struct Wino<2> {
     y[0] = m[0] + m[1] + m[2];
     y[1] = m[1] - m[2] - m[3];
   }
+  // the transposes, for grad-filter: A y and G^T u
+  __device__ static inline void a(const float (&y)[2], float (&m)[4]) {
+    m[0] = y[0];
+    m[1] = y[0] + y[1];
+    m[2] = y[0] - y[1];
+    m[3] = -y[1];
+  }
+  __device__ static inline void gt(const float (&u)[4], float (&f)[3]) {
+    f[0] = u[0] + 0.5f * (u[1] + u[2]);
+    f[1] = 0.5f * (u[1] - u[2]);
+    f[2] = 0.5f * (u[1] + u[2]) + u[3];
+  }
 };
 template <>
 struct Wino<4> {
@@ -407,6 +419,21 @@ struct Wino<4> {
     y[1] = b + 2.f * e;
     y[2] = a + 4.f * c;
     y[3] = b + 8.f * e + m[5];
+  }
+  __device__ static inline void a(const float (&y)[4], float (&m)[6]) {
+    const float e = y[0] + 4.f * y[2], o = 2.f * y[1] + 8.f * y[3];
+    m[0] = y[0];
+    m[1] = (y[0] + y[2]) + (y[1] + y[3]);
+    m[2] = (y[0] + y[2]) - (y[1] + y[3]);
+    m[3] = e + o;
+    m[4] = e - o;
+    m[5] = y[3];
+  }
+  __device__ static inline void gt(const float (&u)[6], float (&f)[3]) {
+    const float s12 = u[1] + u[2], s34 = u[3] + u[4];
+    f[0] = 0.25f * u[0] - (1.f / 6.f) * s12 + (1.f / 24.f) * s34;
+    f[1] = (1.f / 6.f) * (u[2] - u[1]) + (1.f / 12.f) * (u[3] - u[4]);
+    f[2] = (1.f / 6.f) * (s34 - s12) + u[5];
   }
 };
 
@@ -540,88 +567,110 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
 }
 
 // Grad-filter in the same domain: dU[pos][k][c] = sum_t dM[pos][k][t] * V[pos][c][t] with
-// dM = A dY A^T (A = [1 0; 1 1; 1 -1; 0 -1], dY the 2x2 tile of dy, zero beyond the
-// edge) and V the transformed input as in forward; then dw = G^T dU G.
+// dM = A dY A^T (dY the m x m tile of dy, zero beyond the edge) and V the transformed
+// input as in forward; then dw = G^T dU G.  `rows_vec`: Q is a multiple of TILE and dy
+// aligned to a tile row, which is then one 8- or 16-byte load.
+template <int TILE>
 __global__ __launch_bounds__(256) void wino_dy_kernel(const float *__restrict__ dy, float *__restrict__ dM, int K,
                                                      int P, int Q, FastDiv div_tiles, FastDiv div_tw, int T, int Tp,
-                                                     bool pairs) {
+                                                     bool rows_vec) {
+  constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int k = blockIdx.y;
   if (t >= (uint32_t)Tp) return;
-  float y[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  float y[TILE][TILE];
+#pragma unroll
+  for (int a = 0; a < TILE; ++a)
+#pragma unroll
+    for (int b = 0; b < TILE; ++b) y[a][b] = 0.f;
   if (t < (uint32_t)T) {
     uint32_t img, rem, th, tw;
     div_tiles.divmod(t, img, rem);
     div_tw.divmod(rem, th, tw);
-    const int p0 = 2 * (int)th, q0 = 2 * (int)tw;
+    const int p0 = TILE * (int)th, q0 = TILE * (int)tw;
     const float *src = dy + (((int64_t)img * K + k) * P + p0) * Q + q0;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < TILE; ++a) {
       if (p0 + a >= P) break;
-      if (pairs) {
-        const float2 v = *reinterpret_cast<const float2 *>(src + a * Q);
-        y[a][0] = v.x;
-        y[a][1] = v.y;
+      if (rows_vec) {
+        if constexpr (TILE == 2) {
+          const float2 v = *reinterpret_cast<const float2 *>(src + a * Q);
+          y[a][0] = v.x;
+          y[a][1] = v.y;
+        } else {
+          const float4 v = *reinterpret_cast<const float4 *>(src + a * Q);
+          y[a][0] = v.x;
+          y[a][1] = v.y;
+          y[a][2] = v.z;
+          y[a][3] = v.w;
+        }
       } else {
-        y[a][0] = src[a * Q];
-        if (q0 + 1 < Q) y[a][1] = src[a * Q + 1];
+#pragma unroll
+        for (int b = 0; b < TILE; ++b)
+          if (q0 + b < Q) y[a][b] = src[a * Q + b];
       }
     }
   }
-  float r[4][2];
+  float r[A][TILE];  // A dY, column by column
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    r[0][b] = y[0][b];
-    r[1][b] = y[0][b] + y[1][b];
-    r[2][b] = y[0][b] - y[1][b];
-    r[3][b] = -y[1][b];
+  for (int b = 0; b < TILE; ++b) {
+    float col[TILE], o[A];
+#pragma unroll
+    for (int a = 0; a < TILE; ++a) col[a] = y[a][b];
+    Wino<TILE>::a(col, o);
+#pragma unroll
+    for (int i = 0; i < A; ++i) r[i][b] = o[i];
   }
   const int64_t plane_sz = (int64_t)K * Tp;
   float *dst = dM + (int64_t)k * Tp + t;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    dst[(i * 4 + 0) * plane_sz] = r[i][0];
-    dst[(i * 4 + 1) * plane_sz] = r[i][0] + r[i][1];
-    dst[(i * 4 + 2) * plane_sz] = r[i][0] - r[i][1];
-    dst[(i * 4 + 3) * plane_sz] = -r[i][1];
+  for (int i = 0; i < A; ++i) {
+    float o[A];
+    Wino<TILE>::a(r[i], o);
+#pragma unroll
+    for (int j = 0; j < A; ++j) dst[(i * A + j) * plane_sz] = o[j];
   }
 }
 
-// dw[k][c] = G^T (sum over k-splits of dU[split][pos][k][c]) G, G^T = [1 .5 .5 0; 0 .5 -.5 0; 0 .5 .5 1].
-// A workgroup owns 64 filters; lane group g adds the splits of positions 4g..4g+3 in
-// split order (fixed, so the result does not depend on timing), then 64 lanes
-// transform.  KC = K*C.
+// dw[k][c] = G^T (sum over k-splits of dU[split][pos][k][c]) G.  A workgroup owns 64
+// filters; lane group g adds the splits of a quarter of the positions in split order
+// (fixed, so the result does not depend on timing), then 64 lanes transform.  KC = K*C.
+template <int TILE>
 __global__ __launch_bounds__(256) void wino_dfilter_kernel(const float *__restrict__ dU, float *__restrict__ dw,
                                                           int KC, int splits) {
-  __shared__ float u[16][64];
+  constexpr int A = Wino<TILE>::A, POS = A * A, PPG = POS / 4;  // 16 or 36 positions, 4 or 9 per lane group
+  __shared__ float u[POS][64];
   const int lane = threadIdx.x & 63, group = threadIdx.x >> 6;
   const int idx = blockIdx.x * 64 + lane;
   if (idx < KC) {
-    float acc[4];
+    float acc[PPG];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = dU[(int64_t)(group * 4 + j) * KC + idx];
+    for (int j = 0; j < PPG; ++j) acc[j] = dU[(int64_t)(group * PPG + j) * KC + idx];
     for (int sp = 1; sp < splits; ++sp)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] += dU[((int64_t)sp * 16 + group * 4 + j) * KC + idx];
+      for (int j = 0; j < PPG; ++j) acc[j] += dU[((int64_t)sp * POS + group * PPG + j) * KC + idx];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) u[group * 4 + j][lane] = acc[j];
+    for (int j = 0; j < PPG; ++j) u[group * PPG + j][lane] = acc[j];
   }
   __syncthreads();
   if (group != 0 || idx >= KC) return;
-  float r[3][4];
+  float r[3][A];  // G^T dU, column by column
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float u0 = u[j][lane], u1 = u[4 + j][lane], u2 = u[8 + j][lane], u3 = u[12 + j][lane];
-    r[0][j] = u0 + 0.5f * (u1 + u2);
-    r[1][j] = 0.5f * (u1 - u2);
-    r[2][j] = 0.5f * (u1 + u2) + u3;
+  for (int j = 0; j < A; ++j) {
+    float col[A], o[3];
+#pragma unroll
+    for (int i = 0; i < A; ++i) col[i] = u[i * A + j][lane];
+    Wino<TILE>::gt(col, o);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) r[i][j] = o[i];
   }
   float *dst = dw + (int64_t)idx * 9;
 #pragma unroll
   for (int i = 0; i < 3; ++i) {
-    dst[i * 3 + 0] = r[i][0] + 0.5f * (r[i][1] + r[i][2]);
-    dst[i * 3 + 1] = 0.5f * (r[i][1] - r[i][2]);
-    dst[i * 3 + 2] = 0.5f * (r[i][1] + r[i][2]) + r[i][3];
+    float o[3];
+    Wino<TILE>::gt(r[i], o);
+#pragma unroll
+    for (int j = 0; j < 3; ++j) dst[i * 3 + j] = o[j];
   }
 }
 
@@ -756,11 +805,12 @@ struct WinoShape {
   int TH, TW, T, Tp;       // output tiles per image column / row, in total, padded to 4
   size_t u_elems, v_elems, m_elems;  // scratch, each rounded up to 64 floats
 };
-constexpr int kMaxChannelsF4 = 128;  // F(4x4) only up to this many reduction channels (accuracy)
+constexpr int kMaxChannelsF4 = 128;  // F(4x4) only up to this many reduction channels (grad-filter: channels
+                                     // on either side), which bounds its rounding error
 constexpr size_t kMaxWinogradScratch = (size_t)2 << 30;
 
 bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false, int tile = 2) {
-  if (tile != 2 && (tile != 4 || wgrad)) return false;
+  if (tile != 2 && tile != 4) return false;
   w.tile = tile;
   w.positions = (tile + 2) * (tile + 2);
   if (d->R != 3 || d->S != 3 || d->u != 1 || d->v != 1 || d->pad_h > 2 || d->pad_w > 2) return false;
@@ -776,7 +826,7 @@ bool wino_shape(const ConvDesc *d, bool dgrad, WinoShape &w, bool wgrad = false,
   // (grad-filter reduces over the tiles instead and has no such condition)
   if (w.Cr < 1 || w.Cr > 65535 || w.Mo < 1 || w.Mo > 65535) return false;
   if (!wgrad && (w.Cr % 4 != 0 || (dgrad && w.Mo % 4 != 0))) return false;
-  if (tile == 4 && w.Cr > kMaxChannelsF4) return false;
+  if (tile == 4 && (w.Cr > kMaxChannelsF4 || (wgrad && w.Mo > kMaxChannelsF4))) return false;
   w.TH = cdiv(w.out_h, tile);
   w.TW = cdiv(w.out_w, tile);
   const int64_t T = (int64_t)d->N * w.TH * w.TW;
@@ -852,42 +902,63 @@ void consider_winograd(ConvPlan &p, const ConvDesc *d, bool dgrad, double direct
 // Grad-filter in the Winograd domain: batched [K x Tp] * [Tp x C] products, split
 // along the tile index where 16 x tiles leave CUs idle.
 void consider_winograd_wgrad(ConvPlan &p, const ConvDesc *d, double direct_us) {
-  WinoShape w;
-  if (!wino_shape(d, false, w, true)) return;
+  const char *force = getenv("TINYFLOW_WINOGRAD");
+  const int forced = force && *force ? atoi(force) : -1;
+  if (forced == 0) return;
+  const char *cap = getenv("TINYFLOW_WINOGRAD_MAX_TILE");
+  const int max_tile = cap && *cap ? atoi(cap) : 4;
   static const int tiles[3][2] = {{128, 128}, {64, 128}, {64, 64}};
   static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
-  const double out_bytes = 4.0 * 16.0 * d->K * d->C;
-  double best = 1e30;
-  int bm = 64, bn = 64, best_splits = 1;
-  for (auto &t : tiles) {
-    if (t[0] == 128 && d->K <= 64) continue;
-    if (t[1] == 128 && d->C <= 64) continue;
-    for (int splits : cand) {
-      if (splits > 1 && (w.Tp / splits < 64 || splits * out_bytes > 256e6)) continue;
-      const double us = predict_us(d->K, d->C, w.Tp, t[0], t[1], splits, false, false, false, out_bytes, 16);
-      if (us < best) {
-        best = us;
-        bm = t[0];
-        bn = t[1];
-        best_splits = make_geometry(d->K, d->C, w.Tp, bm, bn, splits, stage_depth(bm, bn)).splits;
+  double best_us = 1e30;
+  int best_tile = 0, best_bm = 64, best_bn = 64, best_splits = 1, best_tp = 0;
+  for (int tile : {2, 4}) {
+    // a forced 4 falls back to 2 where the shape does not allow it, so that "forced"
+    // always means some Winograd form for grad-filter
+    WinoShape w;
+    if (!wino_shape(d, false, w, true, tile)) continue;
+    if (forced == 2 && tile != 2) continue;
+    if (forced < 0 && tile > max_tile) continue;
+    const double out_bytes = 4.0 * w.positions * d->K * d->C;
+    double best = 1e30;
+    int bm = 64, bn = 64, splits_of_best = 1;
+    for (auto &t : tiles) {
+      if (t[0] == 128 && d->K <= 64) continue;
+      if (t[1] == 128 && d->C <= 64) continue;
+      for (int splits : cand) {
+        if (splits > 1 && (w.Tp / splits < 64 || splits * out_bytes > 256e6)) continue;
+        const double us = predict_us(d->K, d->C, w.Tp, t[0], t[1], splits, false, false, false, out_bytes, w.positions);
+        if (us < best) {
+          best = us;
+          bm = t[0];
+          bn = t[1];
+          splits_of_best = make_geometry(d->K, d->C, w.Tp, bm, bn, splits, stage_depth(bm, bn)).splits;
+        }
       }
     }
+    const double moved = 4.0 * d->N * ((double)d->C * d->H * d->W + (double)d->K * d->P * d->Q) +
+                         4.0 * (w.v_elems + w.m_elems);
+    const double stream_us = 4.0 * (w.v_elems + w.m_elems) / 5.0e6;
+    double wino_us = std::max(best, stream_us) + moved / 4.0e6 + 6.0;
+    if (forced == 4 && tile == 4) wino_us = 0.0;
+    if (wino_us < best_us) {
+      best_us = wino_us;
+      best_tile = tile;
+      best_bm = bm;
+      best_bn = bn;
+      best_splits = splits_of_best;
+      best_tp = w.Tp;
+    }
   }
-  const double moved = 4.0 * d->N * ((double)d->C * d->H * d->W + (double)d->K * d->P * d->Q) +
-                       4.0 * (w.v_elems + w.m_elems);
-  const double wino_us = best + moved / 4.0e6 + 6.0;
-  const char *force = getenv("TINYFLOW_WINOGRAD");
-  const bool use = force && *force ? atoi(force) != 0 : wino_us < direct_us;
-  if (!use) return;
+  if (best_tile == 0 || (forced < 0 && best_us >= direct_us)) return;
   p.winograd = true;
-  p.wino_tile = 2;
-  p.variant = "wgrad_winograd";
-  p.bm = bm;
-  p.bn = bn;
+  p.wino_tile = best_tile;
+  p.variant = best_tile == 2 ? "wgrad_winograd" : "wgrad_winograd4x4";
+  p.bm = best_bm;
+  p.bn = best_bn;
   p.splits = best_splits;
   p.M = d->K;
   p.N = d->C;
-  p.K = w.Tp;
+  p.K = best_tp;
 }
 
 ConvPlan plan_forward(const ConvDesc *d) {
@@ -1022,11 +1093,11 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
 int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, const float *dy, float *dw,
                        int *memorytoSaving, hipStream_t s) {
   WinoShape w;
-  if (!wino_shape(d, false, w, true)) return -1;
+  if (!wino_shape(d, false, w, true, plan.wino_tile)) return -1;
   const int KC = d->K * d->C;
   const int bk = stage_depth(plan.bm, plan.bn);
   const Geometry g = make_geometry(d->K, d->C, w.Tp, plan.bm, plan.bn, plan.splits, bk);
-  const size_t du_elems = (size_t)g.splits * 16 * KC;
+  const size_t du_elems = (size_t)g.splits * w.positions * KC;
   const size_t bytes = (w.v_elems + w.m_elems + du_elems) * sizeof(float);
   float *V = (float *)device_alloc(bytes);
   if (!V) {
@@ -1035,21 +1106,29 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
   }
   float *dM = V + w.v_elems, *dU = dM + w.m_elems;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
-  hipLaunchKernelGGL(wino_input_kernel<2>, dim3(cdiv(w.Tp, 256), d->C), dim3(256), 0, s, x, V, d->C, d->H, d->W,
-                     div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
-  const bool pairs = d->Q % 2 == 0 && (reinterpret_cast<uintptr_t>(dy) & 7u) == 0;
-  hipLaunchKernelGGL(wino_dy_kernel, dim3(cdiv(w.Tp, 256), d->K), dim3(256), 0, s, dy, dM, d->K, d->P, d->Q,
-                     div_tiles, div_tw, w.T, w.Tp, pairs);
+  const bool rows_vec = d->Q % w.tile == 0 && (reinterpret_cast<uintptr_t>(dy) & (uintptr_t)(4 * w.tile - 1)) == 0;
+  const dim3 block(256);
+  auto transforms_in = [&](auto tile_c) {
+    constexpr int TILE = decltype(tile_c)::value;
+    hipLaunchKernelGGL(wino_input_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
+                       div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
+    hipLaunchKernelGGL(wino_dy_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q,
+                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
+  };
+  if (w.tile == 2) transforms_in(IC<2>{}); else transforms_in(IC<4>{});
   with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     const Batched<Across4<BM, BK>> al{{dM, (uint32_t)((size_t)d->K * w.Tp * 4), w.Tp, d->K, w.Tp, FastDiv(ONE_SEGMENT), 0},
                                       (int64_t)d->K * w.Tp};
     const Batched<Across4<BN, BK>> bl{{V, (uint32_t)((size_t)d->C * w.Tp * 4), w.Tp, d->C, w.Tp, FastDiv(ONE_SEGMENT), 0},
                                       (int64_t)d->C * w.Tp};
-    const StoreBatched ep{{dU, d->C, d->K, d->C, (int64_t)16 * KC}, (int64_t)KC};
-    launch<BM, BN, BK>(al, bl, ep, w.Tp, g, s, 16);
+    const StoreBatched ep{{dU, d->C, d->K, d->C, (int64_t)w.positions * KC}, (int64_t)KC};
+    launch<BM, BN, BK>(al, bl, ep, w.Tp, g, s, w.positions);
   });
-  hipLaunchKernelGGL(wino_dfilter_kernel, dim3(cdiv(KC, 64)), dim3(256), 0, s, (const float *)dU, dw, KC, g.splits);
+  if (w.tile == 2)
+    hipLaunchKernelGGL(wino_dfilter_kernel<2>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
+  else
+    hipLaunchKernelGGL(wino_dfilter_kernel<4>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
   device_free(V);
   return 0;
 }
