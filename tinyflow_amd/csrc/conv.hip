@@ -469,10 +469,13 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
 // V[pos][cr][t] = (B^T d B)[pos]; d is the patch of in[image][cr] whose corner is
 // (TILE*tile_row - pad_h, TILE*tile_col - pad_w), zero outside the image.  One lane per
 // (cr = blockIdx.y, t); columns T..Tp-1 of the padded row are written as zeros.
-template <int TILE>
+// ROW16 (TILE 4 only; W a multiple of 4, `in` 16-byte aligned, pad_w = 1): the four middle
+// columns of a patch row are one aligned 16-byte load.
+template <int TILE, bool ROW16 = false>
 __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
                                                         int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
                                                         int pad_w, int T, int Tp) {
+  static_assert(!ROW16 || TILE == 4, "ROW16 is the 6-wide patch whose columns 1..4 start at a multiple of 4");
   constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int cr = blockIdx.y;
@@ -488,13 +491,30 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
     div_tw.divmod(rem, th, tw);
     const float *plane = in + ((int64_t)img * Cr + cr) * H * W;
     const int h0 = TILE * (int)th - pad_h, w0 = TILE * (int)tw - pad_w;
+    if constexpr (ROW16) {
+      const int wq = w0 + 1;  // = 4 * tw < W
 #pragma unroll
-    for (int i = 0; i < A; ++i)
-#pragma unroll
-      for (int j = 0; j < A; ++j) {
-        const int h = h0 + i, x = w0 + j;
-        if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = plane[h * W + x];
+      for (int i = 0; i < A; ++i) {
+        const int h = h0 + i;
+        if (h < 0 || h >= H) continue;
+        const float *row = plane + h * W + wq;
+        const float4 mid = *reinterpret_cast<const float4 *>(row);
+        if (wq > 0) d[i][0] = row[-1];
+        d[i][1] = mid.x;
+        d[i][2] = mid.y;
+        d[i][3] = mid.z;
+        d[i][4] = mid.w;
+        if (wq + 4 < W) d[i][5] = row[4];
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < A; ++i)
+#pragma unroll
+        for (int j = 0; j < A; ++j) {
+          const int h = h0 + i, x = w0 + j;
+          if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = plane[h * W + x];
+        }
+    }
   }
   float r[A][A];  // B^T d, column by column
 #pragma unroll
@@ -1060,6 +1080,13 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
   auto transforms_in = [&](auto tile_c) {
     constexpr int TILE = decltype(tile_c)::value;
     hipLaunchKernelGGL(wino_filter_kernel<TILE>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad);
+    if constexpr (TILE == 4) {
+      if (w.pad_w == 1 && w.in_w % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0) {
+        hipLaunchKernelGGL((wino_input_kernel<4, true>), igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles,
+                           div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
+        return;
+      }
+    }
     hipLaunchKernelGGL(wino_input_kernel<TILE>, igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles, div_tw,
                        w.pad_h, w.pad_w, w.T, w.Tp);
   };
@@ -1110,8 +1137,14 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
   const dim3 block(256);
   auto transforms_in = [&](auto tile_c) {
     constexpr int TILE = decltype(tile_c)::value;
-    hipLaunchKernelGGL(wino_input_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
-                       div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
+    bool row16 = false;
+    if constexpr (TILE == 4) row16 = d->pad_w == 1 && d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    if (row16)
+      hipLaunchKernelGGL((wino_input_kernel<4, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
+                         div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
+    else
+      hipLaunchKernelGGL(wino_input_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
+                         div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
     hipLaunchKernelGGL(wino_dy_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q,
                        div_tiles, div_tw, w.T, w.Tp, rows_vec);
   };
