@@ -170,24 +170,48 @@ def test_conv_gradients_are_deterministic(rt):
     np.testing.assert_array_equal(outs[0][1], outs[1][1])
 
 
-def test_conv_adjoint_identities_full_size(rt):
-    """<conv(x,w), dy> = <x, dgrad(dy,w)> = <w, wgrad(x,dy)> at a full ResNet-50
-    batch-64 layer shape (too large for the CPU oracle in a unit test)."""
+# ResNet-50 batch-64 layer shapes, one per kernel family: (C, H, K, R, padding, stride)
+FULL_SIZE_LAYERS = [
+    (128, 28, 128, 3, "SAME", 1),    # 3x3, Winograd 4x4 tiles
+    (64, 56, 64, 3, "SAME", 1),
+    (256, 14, 256, 3, "SAME", 1),    # 3x3, Winograd 2x2 tiles
+    (512, 7, 512, 3, "SAME", 1),
+    (64, 56, 256, 1, "VALID", 1),    # 1x1, 16-byte loaders
+    (2048, 7, 512, 1, "VALID", 1),   # 1x1, 49 pixels per image
+    (1024, 14, 2048, 1, "VALID", 2), # 1x1 stride 2: gathered forward, scatter grad-data
+    (3, 224, 64, 7, "SAME", 2),      # stem
+]
+
+
+@pytest.mark.parametrize("layer", FULL_SIZE_LAYERS, ids=lambda l: "x".join(str(v) for v in l))
+def test_conv_adjoint_identities_full_size(rt, layer):
+    """<conv(x,w), dy> = <x, dgrad(dy,w)> = <w, wgrad(x,dy)> at full ResNet-50 batch-64
+    layer shapes (too large for the CPU oracle in a unit test).  The three kernels
+    share no code path beyond the tile engine, so a wrong index in one breaks an
+    identity; each convolution is also checked against the float64 oracle on the
+    first image and a few output channels."""
     from tinyflow_amd import gpu_op, ndarray
+    C, H, K, R, padding, stride = layer
     rng = np.random.RandomState(12)
-    x = rng.normal(0, 1, (64, 128, 28, 28)).astype(np.float32)
-    w = rng.normal(0, 0.03, (128, 128, 3, 3)).astype(np.float32)
-    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", "SAME", 1, 1)
+    x = rng.normal(0, 1, (64, C, H, H)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(2.0 / (C * R * R)), (K, C, R, R)).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", padding, stride, stride)
     dy = rng.normal(0, 1, out_shape).astype(np.float32)
     gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
     gy, gdx, gdw = ndarray.empty(out_shape, rt.ctx), ndarray.empty(x.shape, rt.ctx), ndarray.empty(w.shape, rt.ctx)
     gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream)
     gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream)
     gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream)
-    a = np.vdot(gy.asnumpy().astype(np.float64), dy.astype(np.float64))
+    y = gy.asnumpy()
+    a = np.vdot(y.astype(np.float64), dy.astype(np.float64))
     b = np.vdot(x.astype(np.float64), gdx.asnumpy().astype(np.float64))
     c = np.vdot(w.astype(np.float64), gdw.asnumpy().astype(np.float64))
     assert abs(a - b) <= 1e-4 * abs(a) and abs(a - c) <= 1e-4 * abs(a)
+    pad = O.conv_pad(R, padding)
+    k_some = slice(0, min(K, 8))
+    y_ref = O.conv2d_forward(x[:1].astype(np.float64), w[k_some].astype(np.float64), pad, pad, stride, stride)
+    scale = max(1.0, float(np.abs(y_ref).max()))
+    np.testing.assert_allclose(y[:1, k_some], y_ref, rtol=1e-3, atol=1e-5 * scale)
 
 
 def test_conv_rejects_mismatched_arrays(rt, capfd):
