@@ -1,7 +1,7 @@
 """GPU parity of conv2d forward / grad-data / grad-filter against the oracle.
 
 Tolerance: rtol 1e-3 / atol 1e-5 relative to a float64 evaluation of the
-oracle (the bound BASELINE.json states for conv gradients); the cases cover every
+oracle (the bound this build states for conv gradients); the cases cover every
 filter/stride/padding family of the LeNet, VGG-16 and ResNet-50 configs at
 reduced batch or spatial size, plus ragged sizes that exercise every tile tail.
 """

@@ -1,7 +1,7 @@
 """End-to-end parity of a full training step (forward + backward + SGD) on the GPU
 against the independent layer-by-layer CPU oracle, on identical seeded inputs.
 
-Configs 1 and 2 of BASELINE.json (MLP b128, LeNet-5 b64) run at full size; VGG-16
+The two small benchmark configurations (MLP b128, LeNet-5 b64) run at full size; VGG-16
 and ResNet-50 run structurally complete (all 13 convs / all 16 bottlenecks,
 [3,4,6,3]) at reduced width, image and batch so that the float64 oracle finishes in
 seconds.  Checked per step: the loss, every parameter gradient, every updated

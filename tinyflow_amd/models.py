@@ -192,7 +192,7 @@ def resnet152(rng, batch=128, **kw):
     return resnet(rng, [3, 8, 36, 3], batch, name="resnet152", **kw)
 
 
-# BASELINE configurations: name -> (builder, seed, input distribution)
+# the benchmark configurations: name -> (builder, seed, input distribution)
 CONFIGS = OrderedDict([
     ("mlp", (mlp, 1, "uniform")),
     ("lenet5", (lenet5, 2, "uniform")),
