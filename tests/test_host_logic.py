@@ -68,6 +68,12 @@ def test_conv_out_shape_descriptor(case):
         assert _LIB.DLGpuConvolutionDescribeKernel(lst, which, name, 256, ctypes.byref(flops)) == 0
         assert b" | gemm_kernel<" in name.value
         expect = 2.0 * np.prod(out, dtype=np.float64) * w_shape[1] * w_shape[2] * w_shape[3]
+        variant = name.value.decode().split()[0]
+        if "winograd" in variant:   # flops the batched transformed-domain products execute
+            m = 4 if variant.endswith("4x4") else 2
+            rows, cols = (x_shape[2], x_shape[3]) if which == 1 else (out[2], out[3])
+            tiles = x_shape[0] * -(-rows // m) * -(-cols // m)
+            expect = 2.0 * (m + 2) ** 2 * w_shape[0] * w_shape[1] * tiles
         assert flops.value == expect
 
 
