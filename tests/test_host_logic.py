@@ -77,6 +77,36 @@ def test_conv_out_shape_descriptor(case):
         assert flops.value == expect
 
 
+def _variants(x_shape, w_shape, padding="SAME", stride=1):
+    _, lst = gpu_op.convolution_2d_forward_get_out_shape(x_shape, w_shape, "NCHW", padding, stride, stride)
+    name = ctypes.create_string_buffer(256)
+    out = []
+    for which in range(3):
+        assert _LIB.DLGpuConvolutionDescribeKernel(lst, which, name, 256, None) == 0
+        out.append(name.value.decode().split()[0])
+    return out
+
+
+def test_planner_picks_winograd_forms_by_shape(monkeypatch):
+    """3x3 / stride-1 layers of the ResNet-50 batch-64 configuration: 4x4 tiles up to 128
+    channels, 2x2 tiles above; other filters and strides stay direct; the environment
+    overrides what the cost model would pick."""
+    monkeypatch.delenv("TINYFLOW_WINOGRAD", raising=False)
+    monkeypatch.delenv("TINYFLOW_WINOGRAD_MAX_TILE", raising=False)
+    assert _variants((64, 64, 56, 56), (64, 64, 3, 3)) == ["fwd_winograd4x4", "dgrad_winograd4x4", "wgrad_winograd4x4"]
+    assert _variants((64, 128, 28, 28), (128, 128, 3, 3)) == ["fwd_winograd4x4", "dgrad_winograd4x4", "wgrad_winograd4x4"]
+    assert _variants((64, 256, 14, 14), (256, 256, 3, 3)) == ["fwd_winograd", "dgrad_winograd", "wgrad_winograd"]
+    assert _variants((64, 512, 7, 7), (512, 512, 3, 3)) == ["fwd_winograd", "dgrad_winograd", "wgrad_winograd"]
+    for shapes in (((64, 64, 56, 56), (256, 64, 1, 1), "VALID", 1), ((64, 3, 224, 224), (64, 3, 7, 7), "SAME", 2),
+                   ((64, 128, 56, 56), (128, 128, 3, 3), "SAME", 2)):
+        assert not any("winograd" in v for v in _variants(*shapes))
+    monkeypatch.setenv("TINYFLOW_WINOGRAD_MAX_TILE", "2")
+    assert not any("4x4" in v for v in _variants((64, 128, 28, 28), (128, 128, 3, 3)))
+    assert "fwd_winograd" in _variants((64, 128, 28, 28), (128, 128, 3, 3))
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "0")
+    assert not any("winograd" in v for v in _variants((64, 256, 14, 14), (256, 256, 3, 3)))
+
+
 def test_descriptor_calls_reject_bad_arguments():
     with pytest.raises(RuntimeError):
         gpu_op.convolution_2d_forward_get_out_shape((2, 3, 8, 8), (4, 5, 3, 3), "NCHW", "SAME", 1, 1)  # channel mismatch
