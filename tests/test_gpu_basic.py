@@ -123,6 +123,29 @@ def test_softmax_and_cross_entropy(rt, shape):
     np.testing.assert_allclose(loss.asnumpy(), O.softmax_cross_entropy(y.astype(np.float64), labels), rtol=1e-5)
 
 
+def test_cross_entropy_without_scratch_memory(rt):
+    """More than 16 rows take a two-launch form that needs a small scratch array; with
+    no device memory left the one-launch form runs and gives the same bits."""
+    from tinyflow_amd import gpu_op, ndarray
+    rng = np.random.RandomState(6)
+    shape = (70, 1000)
+    y = rng.uniform(-5, 5, shape).astype(np.float32)
+    labels = np.zeros(shape, np.float32)
+    labels[np.arange(shape[0]), rng.randint(0, shape[1], shape[0])] = 1
+    gy, gl = _gpu(y, rt), _gpu(labels, rt)
+    loss, loss2 = _empty((1,), rt), _empty((1,), rt)
+    gpu_op.softmax_cross_entropy(gy, gl, loss, rt.stream)
+    _, in_use, _ = gpu_op.device_memory_stats()
+    gpu_op.set_device_memory_limit(max(in_use, 1))
+    try:
+        assert isinstance(ndarray.empty((1 << 20,), rt.ctx), int)
+        gpu_op.softmax_cross_entropy(gy, gl, loss2, rt.stream)
+        got = loss2.asnumpy()
+    finally:
+        gpu_op.set_device_memory_limit(0)
+    np.testing.assert_array_equal(got, loss.asnumpy())
+
+
 MM_CASES = [
     # the reference's own cases (tests/test_gpu_op.py:103-131)
     ((500, 700), False, (700, 1000), False),

@@ -171,6 +171,49 @@ __global__ __launch_bounds__(1024) void softmax_xent_kernel(const float *__restr
   }
 }
 
+// The same loss in two launches for more than 16 rows: one wave per row writes the
+// row's term (same arithmetic as above), then one workgroup adds the terms the way
+// the single-workgroup kernel does (wave w takes rows w, w+16, ... in order, the 16
+// wave totals are added in wave order), so both forms give the same bits.
+__global__ __launch_bounds__(kThreads) void softmax_xent_rows_kernel(const float *__restrict__ logits,
+                                                                    const float *__restrict__ labels,
+                                                                    float *__restrict__ row_loss, int rows,
+                                                                    int cols) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const float *x = logits + (int64_t)r * cols;
+  const float *t = labels + (int64_t)r * cols;
+  float m = -INFINITY;
+  for (int c = lane; c < cols; c += 64) m = fmaxf(m, x[c]);
+  m = __shfl(wave_max(m), 0, 64);
+  float s = 0.f;
+  for (int c = lane; c < cols; c += 64) s += expf(x[c] - m);
+  s = __shfl(wave_sum(s), 0, 64);
+  const float log_s = logf(s);
+  float l = 0.f;
+  for (int c = lane; c < cols; c += 64) l -= t[c] * ((x[c] - m) - log_s);
+  l = wave_sum(l);
+  if (lane == 0) row_loss[r] = l;
+}
+
+__global__ __launch_bounds__(1024) void xent_mean_kernel(const float *__restrict__ row_loss, float *__restrict__ out,
+                                                        int rows) {
+  __shared__ float wave_total[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    float total = 0.f;
+    for (int r = wave; r < rows; r += 16) total += row_loss[r];
+    wave_total[wave] = total;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int w = 0; w < 16; ++w) s += wave_total[w];
+    out[0] = s / (float)rows;
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void zero_kernel(float *out, int n) {
   const int i = blockIdx.x * kThreads + threadIdx.x;
   if (i < n) out[i] = 0.f;
@@ -356,9 +399,18 @@ extern "C" int DLGpuSoftmaxCrossEntropy(const DLArrayHandle logits, const DLArra
   TF_REQUIRE(logits->ndim == 2 && same_shape(logits, labels), "logits and labels must be matching 2-D arrays");
   TF_REQUIRE(numel(out) == 1, "output must hold one element");
   hipStream_t s = stream_of(stream);
-  hipLaunchKernelGGL(softmax_xent_kernel, dim3(1), dim3(1024), 0, s, (const float *)logits->data,
-                     (const float *)labels->data, (float *)out->data, (int)logits->shape[0],
-                     (int)logits->shape[1]);
+  const int rows = (int)logits->shape[0], cols = (int)logits->shape[1];
+  // this entry point cannot report exhausted scratch: without it the one-launch form runs
+  float *row_loss = rows > 16 ? (float *)device_alloc((size_t)rows * sizeof(float)) : nullptr;
+  if (row_loss) {
+    hipLaunchKernelGGL(softmax_xent_rows_kernel, dim3(cdiv(rows, kThreads / 64)), dim3(kThreads), 0, s,
+                       (const float *)logits->data, (const float *)labels->data, row_loss, rows, cols);
+    hipLaunchKernelGGL(xent_mean_kernel, dim3(1), dim3(1024), 0, s, (const float *)row_loss, (float *)out->data, rows);
+    device_free(row_loss);
+  } else {
+    hipLaunchKernelGGL(softmax_xent_kernel, dim3(1), dim3(1024), 0, s, (const float *)logits->data,
+                       (const float *)labels->data, (float *)out->data, rows, cols);
+  }
   return finish(s, "DLGpuSoftmaxCrossEntropy");
 }
 
