@@ -74,28 +74,28 @@ def stream_handle(stream_cell):
 # commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
 # --config resnet50 --batch 64 only and are reported as null otherwise.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Along4<128, 16>, StoreNCHW>": 140294777,
-    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Across4<64, 32>>, StoreBatched>": 244570994,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Across4<128, 16>, StoreRowMajor>": 131584554,
-    "gemm_kernel<128, 128, 16, Along4<128, 16>, Along4<128, 16>, StoreNCHW>": 127713322,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Across4<64, 32>, StoreRowMajor>": 223009193,
-    "gemm_kernel<128, 128, 16, Batched<Along4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 137814392,
-    "gemm_kernel<128, 128, 16, Batched<Across4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 137339570,
-    "gemm_kernel<64, 128, 16, Batched<Along4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 218724125,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 218700683,
-    "gemm_kernel<64, 128, 16, Along4<64, 16>, Along4<128, 16>, StoreNCHW>": 227003681,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreScatter>": 225401212,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Across4<128, 16>>, StoreBatched>": 140569765,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 235174727,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126354267,
-    "gemm_kernel<64, 128, 16, Across4<64, 16>, Along4<128, 16>, StoreNCHW>": 206318818,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 288179405,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89389350,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreNCHW>": 132665524,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Along4<64, 32>, StoreNCHW>": 132820280,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171331797,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148064817,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 274261475,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, Along4<128, 16>, StoreNCHW>": 140255494,
+    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Across4<64, 32>>, StoreBatched>": 244568891,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, Across4<128, 16>, StoreRowMajor>": 131578195,
+    "gemm_kernel<128, 128, 16, Along4<128, 16>, Along4<128, 16>, StoreNCHW>": 127729671,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, Across4<64, 32>, StoreRowMajor>": 223005909,
+    "gemm_kernel<128, 128, 16, Batched<Along4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 137813148,
+    "gemm_kernel<128, 128, 16, Batched<Across4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 137332935,
+    "gemm_kernel<64, 128, 16, Batched<Along4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 218723053,
+    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 218696091,
+    "gemm_kernel<64, 128, 16, Along4<64, 16>, Along4<128, 16>, StoreNCHW>": 227003074,
+    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreScatter>": 225304416,
+    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Across4<128, 16>>, StoreBatched>": 140569087,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 235231291,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 126419984,
+    "gemm_kernel<64, 128, 16, Across4<64, 16>, Along4<128, 16>, StoreNCHW>": 206312254,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 288120090,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89347908,
+    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreNCHW>": 132668343,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, Along4<64, 32>, StoreNCHW>": 132813813,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171197226,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148184932,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 1>, StoreRowMajor>": 274188895,
 }
 
 
