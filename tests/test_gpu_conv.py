@@ -78,6 +78,7 @@ WINOGRAD_CASES = [
     ((4, 64, 56, 56, 64, 3, 3, "SAME", 1, 1), True, True),
     ((2, 64, 30, 26, 128, 3, 3, "SAME", 1, 1), True, True),     # extents that are not multiples of 4
     ((4, 512, 7, 7, 512, 3, 3, "SAME", 1, 1), True, True),      # odd extent: half-empty edge tiles
+    ((2, 516, 6, 6, 520, 3, 3, "SAME", 1, 1), True, True),      # more than 512 channels: 2x2 tiles only
     ((2, 64, 14, 14, 256, 3, 3, "SAME", 1, 1), True, True),
     ((3, 8, 5, 5, 12, 3, 3, "SAME", 1, 1), True, True),         # 27 tiles: padded to 28 columns
     ((1, 4, 7, 9, 4, 3, 3, "SAME", 1, 1), True, True),
@@ -95,17 +96,17 @@ WINOGRAD_CASES = [
 @pytest.mark.parametrize("force", ["2", "4"])
 @pytest.mark.parametrize("case,fwd,dgrad", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else str(c))
 def test_conv_winograd_form(rt, monkeypatch, case, fwd, dgrad, force):
-    """F(2x2, 3x3) and F(4x4, 3x3), forced; the latter is limited to 128 reduction channels."""
+    """F(2x2, 3x3) and F(4x4, 3x3), forced; the latter is limited to 512 reduction channels."""
     from tinyflow_amd import gpu_op
     monkeypatch.setenv("TINYFLOW_WINOGRAD", force)
     N, C, H, W, K, R, S, padding, u, v = case
     _, lst = gpu_op.convolution_2d_forward_get_out_shape((N, C, H, W), (K, C, R, S), "NCHW", padding, u, v)
     tag = "winograd4x4" if force == "4" else "winograd "
-    assert (tag in _describe(lst, 0)) == (fwd and (force == "2" or C <= 128))
-    assert (tag in _describe(lst, 1)) == (dgrad and (force == "2" or K <= 128))
+    assert (tag in _describe(lst, 0)) == (fwd and (force == "2" or C <= 512))
+    assert (tag in _describe(lst, 1)) == (dgrad and (force == "2" or K <= 512))
     # grad-filter reduces over the tiles: no condition on the channel counts for 2x2 tiles,
-    # which also stand in where 4x4 tiles are not allowed (more than 128 channels)
-    wtag = "wgrad_winograd4x4" if force == "4" and C <= 128 and K <= 128 else "wgrad_winograd "
+    # which also stand in where 4x4 tiles are not allowed (more than 512 channels)
+    wtag = "wgrad_winograd4x4" if force == "4" and C <= 512 and K <= 512 else "wgrad_winograd "
     assert (wtag in _describe(lst, 2)) == (u == 1 and v == 1)
     _check_conv_case(rt, case)
     monkeypatch.setenv("TINYFLOW_WINOGRAD", "0")

