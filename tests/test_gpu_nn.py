@@ -24,6 +24,8 @@ POOL_CASES = [
     ((4, 64, 112, 112), "max", 1, 1, 2, 2, 3, 3),   # ResNet stem pool (pad 1)
     ((4, 64, 112, 112), "max", 0, 0, 2, 2, 3, 3),   # the reference graph's pad 0 variant
     ((8, 2048, 7, 7), "mean", 0, 0, 1, 1, 7, 7),    # global average pool
+    ((3, 5, 4, 6), "mean", 0, 0, 1, 1, 4, 6),       # global, 15 planes of 24 values
+    ((300, 3, 6, 6), "mean", 0, 0, 2, 2, 6, 6),     # global whatever the stride; several workgroups
     ((3, 5, 13, 9), "max", 1, 0, 2, 1, 3, 2),
     ((3, 5, 13, 9), "mean", 1, 1, 2, 2, 3, 3),
     ((2, 3, 8, 8), "max", 0, 0, 1, 1, 1, 1),

@@ -324,6 +324,40 @@ __global__ __launch_bounds__(kThreads) void pool_max_backward_tile_kernel(const 
   }
 }
 
+// Global pooling (the window is the whole, unpadded plane; one output per plane), mean
+// mode: a workgroup stages `planes` consecutive planes -- one contiguous run of memory --
+// in LDS with coalesced loads, then one lane per plane adds its HW values in the order
+// of the general kernel (same bits).  `planes` * HW <= kGlobalFloats.
+constexpr int kGlobalFloats = 8192;
+__global__ __launch_bounds__(kThreads) void global_mean_forward_kernel(const float *__restrict__ x,
+                                                                      float *__restrict__ y, int HW, int planes,
+                                                                      int total_planes) {
+  __shared__ float xs[kGlobalFloats];
+  const int first = blockIdx.x * planes;
+  const int here = min(planes, total_planes - first);
+  const float *src = x + (int64_t)first * HW;
+  for (int i = threadIdx.x; i < here * HW; i += kThreads) xs[i] = src[i];
+  __syncthreads();
+  if ((int)threadIdx.x < here) {
+    float acc = 0.f;
+    for (int i = 0; i < HW; ++i) acc += xs[threadIdx.x * HW + i];
+    y[first + threadIdx.x] = acc / (float)HW;
+  }
+}
+
+// its backward: every element of a plane receives dy[plane] / HW
+__global__ __launch_bounds__(kThreads) void global_mean_backward_kernel(const float *__restrict__ dy,
+                                                                       float *__restrict__ dx, FastDiv div_hw,
+                                                                       float hw, uint32_t total) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < total) dx[i] = dy[div_hw.div(i)] / hw;
+}
+
+bool is_global_mean(const PoolDesc *d) {
+  return d->mode != 0 && d->fh == d->H && d->fw == d->W && d->pad_h == 0 && d->pad_w == 0 && d->P == 1 && d->Q == 1 &&
+         d->H * d->W <= kGlobalFloats;
+}
+
 int grid_for(int64_t n) {
   int64_t blocks = (n + kThreads - 1) / kThreads;
   const int64_t cap = (int64_t)num_cus() * 32;
@@ -393,6 +427,12 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
   if (total == 0) return 0;
   TF_REQUIRE(numel(input) < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   const PoolParams pp = params_of(d);
+  if (is_global_mean(d)) {
+    const int HW = d->H * d->W, planes = std::min(kThreads, kGlobalFloats / HW);
+    hipLaunchKernelGGL(global_mean_forward_kernel, dim3(cdiv(total, planes)), dim3(kThreads), 0, s,
+                       (const float *)input->data, (float *)output->data, HW, planes, (int)total);
+    return finish(s, "DLGpuPooling2DForward");
+  }
   if (d->mode == 0)
     hipLaunchKernelGGL(pool_forward_kernel<true>, dim3(grid_for(total)), dim3(kThreads), 0, s,
                        (const float *)input->data, (float *)output->data, pp, (uint32_t)total);
@@ -418,6 +458,13 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
   if (total == 0) return 0;
   TF_REQUIRE(total < ((int64_t)1 << 31), "tensors of 2^31 elements or more are not supported");
   const PoolParams pp = params_of(d);
+  if (is_global_mean(d)) {
+    const int HW = d->H * d->W;
+    hipLaunchKernelGGL(global_mean_backward_kernel, dim3(cdiv(total, kThreads)), dim3(kThreads), 0, s,
+                       (const float *)doutput->data, (float *)dinput->data, FastDiv((uint32_t)HW), (float)HW,
+                       (uint32_t)total);
+    return finish(s, "DLGpuPooling2DBackward");
+  }
   if (d->mode == 0) {
     TF_REQUIRE(d->fh * d->fw < 255, "max-pool windows of 255 or more taps are not supported");
     const int tiles_h = cdiv(d->H, kTileH), tiles_w = cdiv(d->W, kTileW);
