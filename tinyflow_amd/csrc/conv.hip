@@ -482,9 +482,10 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
 // V[pos][cr][t] = (B^T d B)[pos]; d is the patch of in[image][cr] whose corner is
 // (TILE*tile_row - pad_h, TILE*tile_col - pad_w), zero outside the image.  One lane per
 // (cr = blockIdx.y, t); columns T..Tp-1 of the padded row are written as zeros.
-// ROW16 (TILE 4 only; W a multiple of 4, `in` 16-byte aligned, pad_w = 1): the four middle
-// columns of a patch row are one aligned 16-byte load.
-template <int TILE, bool ROW16 = false>
+// ROW16 (TILE 4 only; pad_w = 1): the four middle columns of a patch row start at a
+// multiple of 4 and are fetched as one 16-byte load (W a multiple of 4, `in` 16-byte
+// aligned) or, with `halves`, as two 8-byte loads (W even, `in` 8-byte aligned).
+template <int TILE, bool ROW16 = false, bool HALVES = false>
 __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
                                                         int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
                                                         int pad_w, int T, int Tp) {
@@ -511,12 +512,23 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
         const int h = h0 + i;
         if (h < 0 || h >= H) continue;
         const float *row = plane + h * W + wq;
-        const float4 mid = *reinterpret_cast<const float4 *>(row);
         if (wq > 0) d[i][0] = row[-1];
-        d[i][1] = mid.x;
-        d[i][2] = mid.y;
-        d[i][3] = mid.z;
-        d[i][4] = mid.w;
+        if constexpr (HALVES) {  // the last tile of a row may hold only two columns
+          const float2 lo = *reinterpret_cast<const float2 *>(row);
+          d[i][1] = lo.x;
+          d[i][2] = lo.y;
+          if (wq + 2 < W) {
+            const float2 hi = *reinterpret_cast<const float2 *>(row + 2);
+            d[i][3] = hi.x;
+            d[i][4] = hi.y;
+          }
+        } else {
+          const float4 mid = *reinterpret_cast<const float4 *>(row);
+          d[i][1] = mid.x;
+          d[i][2] = mid.y;
+          d[i][3] = mid.z;
+          d[i][4] = mid.w;
+        }
         if (wq + 4 < W) d[i][5] = row[4];
       }
     } else {
@@ -1099,6 +1111,11 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
                            div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
         return;
       }
+      if (w.pad_w == 1 && w.in_w % 2 == 0 && (reinterpret_cast<uintptr_t>(in) & 7u) == 0) {
+        hipLaunchKernelGGL((wino_input_kernel<4, true, true>), igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w,
+                           div_tiles, div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
+        return;
+      }
     }
     hipLaunchKernelGGL(wino_input_kernel<TILE>, igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles, div_tw,
                        w.pad_h, w.pad_w, w.T, w.Tp);
@@ -1150,11 +1167,17 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
   const dim3 block(256);
   auto transforms_in = [&](auto tile_c) {
     constexpr int TILE = decltype(tile_c)::value;
-    bool row16 = false;
-    if constexpr (TILE == 4) row16 = d->pad_w == 1 && d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    bool row16 = false, halves = false;
+    if constexpr (TILE == 4) {
+      row16 = d->pad_w == 1 && d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+      halves = !row16 && d->pad_w == 1 && d->W % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0;
+    }
     if (row16)
       hipLaunchKernelGGL((wino_input_kernel<4, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
                          div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
+    else if (halves)
+      hipLaunchKernelGGL((wino_input_kernel<4, true, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H,
+                         d->W, div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
     else
       hipLaunchKernelGGL(wino_input_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
                          div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
