@@ -74,29 +74,29 @@ def stream_handle(stream_cell):
 # commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
 # --config resnet50 --batch 64 only and are reported as null otherwise.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Across4<64, 32>>, StoreBatched>": 210405898,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Along4<128, 16>, StoreNCHW>": 140303123,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Across4<128, 16>, StoreRowMajor>": 131541881,
-    "gemm_kernel<128, 128, 16, Along4<128, 16>, Along4<128, 16>, StoreNCHW>": 127697880,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Across4<64, 32>, StoreRowMajor>": 222993961,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 179934683,
-    "gemm_kernel<64, 128, 16, Batched<Along4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 179564391,
-    "gemm_kernel<64, 128, 16, Along4<64, 16>, Along4<128, 16>, StoreNCHW>": 226992850,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreScatter>": 225298824,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 235159164,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 127570466,
-    "gemm_kernel<64, 64, 32, Batched<Along4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207723020,
-    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207656357,
-    "gemm_kernel<64, 128, 16, Across4<64, 16>, Along4<128, 16>, StoreNCHW>": 206306290,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 287984298,
-    "gemm_kernel<128, 128, 16, Batched<Along4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134839405,
-    "gemm_kernel<128, 128, 16, Batched<Across4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134755133,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89312242,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreNCHW>": 132615140,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Across4<128, 16>>, StoreBatched>": 151162418,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Along4<64, 32>, StoreNCHW>": 132804821,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171319657,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148429092,
+    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Across4<64, 32>>, StoreBatched>": 210391435,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, Along4<128, 16>, StoreNCHW>": 140242015,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, Across4<128, 16>, StoreRowMajor>": 131504118,
+    "gemm_kernel<128, 128, 16, Along4<128, 16>, Along4<128, 16>, StoreNCHW>": 127779549,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, Across4<64, 32>, StoreRowMajor>": 222997758,
+    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 180019254,
+    "gemm_kernel<64, 128, 16, Batched<Along4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 179452610,
+    "gemm_kernel<64, 128, 16, Along4<64, 16>, Along4<128, 16>, StoreNCHW>": 227002849,
+    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreScatter>": 225359672,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 235497575,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 127443020,
+    "gemm_kernel<64, 64, 32, Batched<Along4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207728188,
+    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207656627,
+    "gemm_kernel<64, 128, 16, Across4<64, 16>, Along4<128, 16>, StoreNCHW>": 206299823,
+    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 288039008,
+    "gemm_kernel<128, 128, 16, Batched<Along4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134844673,
+    "gemm_kernel<128, 128, 16, Batched<Across4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134751909,
+    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89372689,
+    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreNCHW>": 132705032,
+    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Across4<128, 16>>, StoreBatched>": 151099603,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, Along4<64, 32>, StoreNCHW>": 132824043,
+    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171230225,
+    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148485080,
 }
 
 
