@@ -65,9 +65,17 @@ int DLArrayFree(DLArrayHandle handle);
 
 /* Copy between host/device arrays of equal byte size.  stream == NULL: fully
  * synchronous.  Otherwise `stream` points at a stream cell; the copy runs on
- * that stream and the call returns after it completed.
+ * that stream, ordered after everything enqueued on the kernel streams, and the
+ * call returns after it completed -- except a device-to-device copy on a stream
+ * that op entry points launch on, which stays asynchronous (later ops on that
+ * stream are ordered behind it).
  * ref: c_runtime_api.h:70-71, c_runtime_api.cc:130-164 */
 int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream);
+
+/* No counterpart in the reference: the rule above as a pure function, so that it
+ * can be checked without a GPU.  kind: 0 host->device, 1 device->host,
+ * 2 device->device; returns 1 when DLArrayCopyFromTo waits for the copy. */
+int DLArrayCopyWaitsForCompletion(int kind, int stream_runs_kernels, int sync_every_op);
 
 /* No counterpart in the reference.  Host -> device copy into an array that came from
  * DLArrayAlloc and has not been used since (the prefetch of the swap path): only

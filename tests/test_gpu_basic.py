@@ -231,6 +231,30 @@ def test_copy_with_stream_and_d2d(rt):
     np.testing.assert_array_equal(c.asnumpy(), x)
 
 
+def test_d2d_copy_on_a_side_stream_is_complete_on_return(rt):
+    """A device-to-device copy on a stream no op launches on, followed at once by a
+    kernel on the compute stream that reads the destination and by a release and
+    reuse of the source: the call has to have waited for the copy."""
+    from tinyflow_amd import gpu_op, ndarray
+    side = gpu_op.create_cudaStream()
+    rng = np.random.RandomState(8)
+    n = 64 << 20   # 256 MiB: long enough that an unfinished copy would be caught
+    x = rng.normal(0, 1, (n,)).astype(np.float32)
+    for _ in range(3):
+        src = _gpu(x, rt)
+        dst = _empty((n,), rt)
+        out = _empty((n,), rt)
+        gpu_op.array_set(dst, 0.0, rt.stream)
+        src.copyto(dst, side)
+        gpu_op.matrix_elementwise_multiply_by_const(dst, 2.0, out, rt.stream)   # reads dst on the compute stream
+        src.free_gpu()
+        clobber = _empty((n,), rt)                                               # may take src's storage
+        gpu_op.array_set(clobber, -7.0, rt.stream)
+        np.testing.assert_array_equal(out.asnumpy(), x * np.float32(2.0))
+        np.testing.assert_array_equal(dst.asnumpy(), x)
+    gpu_op.destroy_cudaStream(side)
+
+
 def test_empty_tensors_are_accepted_everywhere(rt):
     """Zero-element operands: every entry point returns success and launches nothing
     (an empty batch, a layer with no outputs)."""

@@ -42,6 +42,22 @@ def test_library_exports_every_declared_symbol():
     assert not missing, "declared in include/c_runtime_api.h but not exported: %s" % missing
 
 
+def test_streamed_copy_waits_unless_the_stream_orders_its_readers():
+    """DLArrayCopyFromTo with a stream: copies that touch host memory always wait (the
+    reference syncs after every streamed copy, src/c_runtime_api.cc:148-158); a
+    device-to-device copy may stay asynchronous only on a stream that op entry points
+    launch on, because nothing else would order a later reader behind it."""
+    H2D, D2H, D2D = 0, 1, 2
+    f = _LIB.DLArrayCopyWaitsForCompletion
+    for runs_kernels in (0, 1):
+        for sync in (0, 1):
+            assert f(H2D, runs_kernels, sync) == 1
+            assert f(D2H, runs_kernels, sync) == 1
+    assert f(D2D, 1, 0) == 0      # compute stream: later kernels are enqueued behind the copy
+    assert f(D2D, 0, 0) == 1      # copy-only side stream: wait, as the reference does
+    assert f(D2D, 1, 1) == 1 and f(D2D, 0, 1) == 1
+
+
 def test_struct_layout_matches_the_abi():
     """DLContext is 8 bytes, DLArray 32 (src/dlarray.h:21-52)."""
     from tinyflow_amd import ndarray

@@ -464,8 +464,26 @@ class SwapExecutor(object):
         self.Variable_node_np_value = values
 
     def close(self):
-        self.offloader.stop()
-        self.prefetcher.stop()
+        """Stops the two copy workers and gives their streams, the compute stream and
+        the handles back to the library.  Arrays already returned stay valid."""
+        if self.cudaStream is None:
+            return
+        for worker in (self.offloader, self.prefetcher):
+            worker.stop()
+        for worker in (self.offloader, self.prefetcher):
+            worker.join(30.0)
+            if not worker.is_alive():
+                gpu_op.destroy_cudaStream(worker.stream)
+        stream, self.cudaStream = self.cudaStream, None
+        gpu_op.destroy_cudnnHandle(self.cudnnHandle)
+        gpu_op.destroy_cublasHandle(self.cublasHandle)
+        gpu_op.destroy_cudaStream(stream)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:   # interpreter shutdown: the library may already be gone
+            pass
 
     # ------------------------------------------------------------------ set-up
 
@@ -552,7 +570,8 @@ class SwapExecutor(object):
                 break
             if self.offloader.pending or self.prefetcher.pending:
                 waited = time.perf_counter()
-                self.offloader.wait_for_progress(0.05)
+                # wait on a worker that has something queued: the other one returns at once
+                (self.offloader if self.offloader.pending else self.prefetcher).wait_for_progress(0.05)
                 self.stats["alloc_wait_seconds"] = (self.stats.get("alloc_wait_seconds", 0.0)
                                                     + time.perf_counter() - waited)
                 continue

@@ -133,6 +133,25 @@ class TrainExecutor(object):
         """Device array currently holding ``node`` (any node of the step graph)."""
         return self.node_to_arr_map[node]
 
+    def close(self):
+        """Gives the stream and the two handles back to the library (waits for the
+        stream first).  The library orders copies and storage reuse against every
+        stream that has run kernels, so an executor that is done should not leave
+        its stream registered.  Arrays already returned stay valid."""
+        if self.cudaStream is None:
+            return
+        stream, self.cudaStream = self.cudaStream, None
+        self._plan = None
+        gpu_op.destroy_cudnnHandle(self.cudnnHandle)
+        gpu_op.destroy_cublasHandle(self.cublasHandle)
+        gpu_op.destroy_cudaStream(stream)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:   # interpreter shutdown: the library may already be gone
+            pass
+
 
 def find_bn_relu_pairs(topo_order, outputs):
     """Batch norms that can be evaluated together with the ReLU that follows them.

@@ -509,7 +509,26 @@ int wait_for_other_streams(hipStream_t s) {
   return 0;
 }
 
+// True when an op entry point has launched on `s`: later kernels of the step are
+// then enqueued behind whatever is put on `s` now.
+bool stream_runs_kernels(hipStream_t s) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  for (auto &rec : r.streams)
+    if (rec.stream == s) return rec.runs_kernels;
+  return false;
+}
+
 }  // namespace
+
+// Decision table of the streamed copy, exported for the host-logic test: does
+// DLArrayCopyFromTo wait for the copy before it returns?  kind: 0 host->device,
+// 1 device->host, 2 device->device.
+extern "C" int DLArrayCopyWaitsForCompletion(int kind, int stream_runs_kernels_flag, int sync_every_op_flag) {
+  if (kind != 2) return 1;                  // host memory must be readable / reusable on return
+  if (sync_every_op_flag) return 1;
+  return stream_runs_kernels_flag ? 0 : 1;  // a copy-only stream orders nothing behind the copy
+}
 
 extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
   TF_REQUIRE(from && to && from->data && to->data, "null array");
@@ -532,9 +551,14 @@ extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamH
   hipStream_t s = reinterpret_cast<hipStream_t>(*reinterpret_cast<void **>(stream));
   if (wait_for_other_streams(s) != 0) return -1;
   TF_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, s));
-  // Host memory must be readable / reusable on return.  A device-to-device copy
-  // is only ever observed by later stream-ordered work, so it stays asynchronous.
-  if (kind != hipMemcpyDeviceToDevice || sync_every_op()) TF_HIP(hipStreamSynchronize(s));
+  // Host memory must be readable / reusable on return.  A device-to-device copy on
+  // the stream the kernels run on is only ever observed by later work of that
+  // stream, so it stays asynchronous; on any other stream nothing would order the
+  // readers of `to` (or a reuse of `from`'s storage after DLArrayFree) behind the
+  // copy, so the call waits for it as the reference does (src/c_runtime_api.cc:148-158).
+  const int kind_code = kind == hipMemcpyHostToDevice ? 0 : kind == hipMemcpyDeviceToHost ? 1 : 2;
+  if (DLArrayCopyWaitsForCompletion(kind_code, stream_runs_kernels(s) ? 1 : 0, sync_every_op() ? 1 : 0))
+    TF_HIP(hipStreamSynchronize(s));
   return 0;
 }
 
