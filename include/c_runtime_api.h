@@ -144,6 +144,16 @@ int DLGpuBroadcastToBackward1(const DLArrayHandle input, DLArrayHandle output);
 /* out[j] = sum_i in[i, j].  ref: c_runtime_api.h:101, gpu_op.cu:179-189, 950-963 */
 int DLGpuReduceSumAxisZero(const DLArrayHandle input, DLArrayHandle output);
 
+/* The same column sums with the same bits, for callers that cannot allocate
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  The per-chunk partial sums live
+ * in a 2 MiB device array built into the library (one copy per GPU, held until
+ * the process ends) instead of pool memory; no hipMalloc / hipFree / memset is
+ * issued.  A shape whose partial sums do not fit returns -1 with a message (2 MiB
+ * covers every shape the chunking rule produces for this reduction).  Calls on
+ * one GPU share the array: calls that overlap on different streams race. */
+int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle input, DLArrayHandle output, void **stream);
+
 /* ref: c_runtime_api.h:110-141, gpu_op.cu:193-219, 1090-1164 */
 int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB,
                               DLArrayHandle output, void **stream);

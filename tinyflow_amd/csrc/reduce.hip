@@ -10,6 +10,8 @@
 // :237-302, 1235-1287 (softmax, softmax cross entropy).
 #include "internal.h"
 
+#include <mutex>
+
 using namespace tf;
 
 namespace {
@@ -226,8 +228,13 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // that cannot report exhausted scratch passes scratch_bytes == nullptr: the sum
 // then runs as a single chunk, which needs no scratch (slower on short outputs,
 // and the additions associate differently than in the chunked run).
+//
+// `fixed` / `fixed_bytes` name a caller-owned scratch area to use instead of the
+// pool (the entry point that must not allocate): the chunking is the same, so the
+// result has the same bits; when the partial sums do not fit, -2 is returned and
+// nothing is launched.
 int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hipStream_t s,
-               size_t *scratch_bytes, const char *what) {
+               size_t *scratch_bytes, const char *what, float *fixed = nullptr, size_t fixed_bytes = 0) {
   if (B == 0) return 0;
   if (A > INT32_MAX || B > INT32_MAX || C > INT32_MAX) {
     fprintf(stderr, "[tinyflow_amd] %s: extents of 2^31 or more are not supported\n", what);
@@ -252,7 +259,15 @@ int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hip
   float *partial = out;
   if (chunks > 1) {
     const size_t bytes = (size_t)chunks * (size_t)B * sizeof(float);
-    partial = (float *)device_alloc(bytes);
+    if (fixed) {
+      if (bytes > fixed_bytes) {
+        if (scratch_bytes) *scratch_bytes = bytes;
+        return -2;
+      }
+      partial = fixed;
+    } else {
+      partial = (float *)device_alloc(bytes);
+    }
     if (!partial) {
       if (scratch_bytes) {
         *scratch_bytes = bytes;
@@ -276,7 +291,7 @@ int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hip
   if (chunks > 1) {
     hipLaunchKernelGGL(finalsum_kernel, dim3(cdiv(B, kThreads)), dim3(kThreads), 0, s, partial, out, (int)B,
                        chunks);
-    device_free(partial);  // stream-ordered reuse: later users are enqueued behind finalsum
+    if (!fixed) device_free(partial);  // stream-ordered reuse: later users are enqueued behind finalsum
   }
   return finish(s, what);
 }
@@ -292,6 +307,56 @@ extern "C" int DLGpuReduceSumAxisZero(const DLArrayHandle in, DLArrayHandle out)
   // 1-D input (n,) -> (1,): one column of n rows
   return reduce_abc((const float *)in->data, (float *)out->data, A, in->ndim == 1 ? 1 : B, 1, nullptr, nullptr,
                     "DLGpuReduceSumAxisZero");
+}
+
+// ---- the entry point that allocates nothing -----------------------------------
+// The column sums' per-chunk partials live in a file-scope device array instead of
+// pool memory.  Each device holds its own copy of the array at its own address, so
+// the address is looked up once per device (hipGetSymbolAddress with that device
+// current) and that pointer, never the symbol, is what the kernels receive.
+constexpr size_t kFixedScratchBytes = 2u << 20;
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 16;
+std::mutex fixed_mu;
+float *fixed_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device; nullptr (with a message) on failure.
+float *fixed_scratch_of_current_device(const char *what) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fprintf(stderr, "[tinyflow_amd] %s: no current device (or device index above %d)\n", what, kMaxDevices - 1);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> g(fixed_mu);
+  if (!fixed_ptr[dev]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fprintf(stderr, "[tinyflow_amd] %s: hipGetSymbolAddress failed: %s\n", what, hipGetErrorString(e));
+      return nullptr;
+    }
+    fixed_ptr[dev] = (float *)p;
+  }
+  return fixed_ptr[dev];
+}
+}  // namespace
+
+extern "C" int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
+  TF_REQUIRE(in->ndim >= 1, "input needs at least one dim");
+  const int64_t A = in->shape[0];
+  const int64_t B = numel(in) / (A > 0 ? A : 1);
+  TF_REQUIRE(numel(out) == (in->ndim == 1 ? 1 : B), "output must be input.shape[1:]");
+  float *fixed = fixed_scratch_of_current_device("DLGpuReduceSumAxisZeroNoAlloc");
+  if (!fixed) return -1;
+  size_t want = 0;
+  const int rc = reduce_abc((const float *)in->data, (float *)out->data, A, in->ndim == 1 ? 1 : B, 1,
+                            stream_of(stream), &want, "DLGpuReduceSumAxisZeroNoAlloc", fixed, kFixedScratchBytes);
+  TF_REQUIRE(rc != -2, "partial sums need %zu bytes, the built-in scratch area holds %zu", want,
+             kFixedScratchBytes);
+  return rc;
 }
 
 extern "C" int DLGpuBroadcastToBackward0(const DLArrayHandle in, DLArrayHandle out) {

@@ -101,6 +101,13 @@ def reduce_sum_axis_zero(in_arr, out_arr):
     check_call(_LIB.DLGpuReduceSumAxisZero(in_arr.handle, out_arr.handle))
 
 
+def reduce_sum_axis_zero_no_alloc(in_arr, out_arr, cudaStream):
+    """reduce_sum_axis_zero for callers that cannot allocate: partial sums go to a
+    device array built into the library (extension: no counterpart in the reference)"""
+    _nd_args(in_arr, out_arr)
+    check_call(_LIB.DLGpuReduceSumAxisZeroNoAlloc(in_arr.handle, out_arr.handle, cudaStream))
+
+
 def matrix_elementwise_add(matA, matB, matC, cudaStream):
     _nd_args(matA, matB, matC)
     check_call(_LIB.DLGpuMatrixElementwiseAdd(matA.handle, matB.handle, matC.handle, cudaStream))
