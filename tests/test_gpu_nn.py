@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from oracle import ops as O
+import parity
 
 pytestmark = pytest.mark.gpu
 
@@ -149,6 +150,9 @@ BN_SHAPES = [(64, 64, 28, 28), (32, 16, 7, 9), (5, 3, 4, 4), (128, 8, 6, 6), (20
              (64, 256, 56, 56)]   # the last one: the largest ResNet-50 b64 activation
 
 
+K_BN = 3.0
+
+
 @pytest.mark.parametrize("shape", BN_SHAPES, ids=str)
 @pytest.mark.parametrize("mode", ["pre_activation", "spatial"])
 def test_batch_norm(rt, shape, mode):
@@ -168,6 +172,13 @@ def test_batch_norm(rt, shape, mode):
     np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-3, atol=2e-5)
     scale = max(1.0, float(np.abs(dx_ref).max()))
     np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-3, atol=2e-5 * scale)
+    # against what a numpy fp32 executor gives on the same inputs: the HIP error may be
+    # at most K_BN times the float32 oracle's own distance from the float64 one
+    y32, mean32, istd32 = O.batch_norm_forward(x, mode)
+    dx32 = O.batch_norm_backward(x, dy, mode, mean32, istd32)
+    assert y32.dtype == dx32.dtype == np.float32
+    parity.compare(gy.asnumpy(), y_ref, y32, "batch norm forward, %s" % mode, "bn fwd %s %s" % (shape, mode), K_BN)
+    parity.compare(gdx.asnumpy(), dx_ref, dx32, "batch norm backward, %s" % mode, "bn bwd %s %s" % (shape, mode), K_BN)
     # invariants of the batch-norm gradient per statistic group:
     #   sum(dx) = 0 and sum(dx * xhat) = istd/m * sum(dy*xhat) * (m - sum(xhat^2))
     # (the second is 0 only in the limit eps -> 0, because sum(xhat^2) = m*var/(var+eps))
@@ -183,6 +194,37 @@ def test_batch_norm(rt, shape, mode):
     # a second backward without a forward is refused (statistics were consumed)
     with pytest.raises(RuntimeError):
         gpu_op.bn_backward(gx, gdy, gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["pre_activation", "spatial"])
+def test_batch_norm_with_mean_far_from_zero(rt, mode):
+    """Statistics whose mean is a thousand standard deviations from zero (mean about
+    100, std about 0.1): a variance computed as E[x^2] - mean^2 in fp32 would be lost to
+    cancellation.  Forward and backward against the float64 oracle; the fp32 CPU oracle
+    (two-pass variance) is the yardstick for the error."""
+    from tinyflow_amd import gpu_op, ndarray
+    shape = (32, 24, 14, 14)
+    rng = np.random.RandomState(29)
+    offset = rng.choice([-1.0, 1.0], (1,) + shape[1:]) * rng.uniform(80, 120, (1,) + shape[1:])
+    x = (offset + rng.normal(0, 1, shape) * rng.uniform(0.05, 0.2, (1,) + shape[1:])).astype(np.float32)
+    dy = rng.normal(0, 1, shape).astype(np.float32)
+    mean_p, var_p, lst = gpu_op.bn_get_cudnnlist(shape, "NCHW", mode)
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    assert gpu_op.bn_forward(gx, gy, mode, 0, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.bn_backward(gx, gdy, gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    y_ref, mean, istd = O.batch_norm_forward(x64, mode)
+    dx_ref = O.batch_norm_backward(x64, dy64, mode, mean, istd)
+    y32, mean32, istd32 = O.batch_norm_forward(x, mode)
+    dx32 = O.batch_norm_backward(x, dy, mode, mean32, istd32)
+    # x itself carries 100 * 2^-24 = 6e-6 of rounding against a spread of 0.1: the
+    # normalised values are only defined to about 1e-4, whoever computes them
+    np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-3, atol=2e-3)
+    np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-3, atol=2e-3 * float(np.abs(dx_ref).max()))
+    parity.compare(gy.asnumpy(), y_ref, y32, "batch norm forward, %s, |mean| >> std" % mode, "bn fwd offset", K_BN)
+    parity.compare(gdx.asnumpy(), dx_ref, dx32, "batch norm backward, %s, |mean| >> std" % mode, "bn bwd offset", K_BN)
 
 
 # ------------------------------------------------------- dropout, concatenation

@@ -1,0 +1,101 @@
+"""ResNet-50 at its real width (64 ... 2048 channels) and resolution (3x224x224),
+batch 8, one training step end to end against the CPU oracle.
+
+The reduced networks of tests/test_gpu_train_step.py never reach the channel counts
+and map sizes the benchmark runs (and therefore neither the tile shapes, split
+counts nor the Winograd forms the launch planner picks there).  Here the graph is
+the benchmark's; only the batch is 8 so that the float64 oracle finishes in seconds.
+Run twice: with the planner's own choices, and with F(4x4, 3x3) forced on every
+eligible 3x3 convolution, grad-data and grad-filter -- the form the planner takes
+for all four 3x3 stages at batch 64.
+
+Checked: the loss within rtol 1e-4 of the float64 oracle; every parameter gradient
+in relative L2 within max(5e-2, 3 x the float32 CPU oracle's own distance from the
+float64 one).  A 50-layer batch-normalised stack at batch 8 amplifies rounding (a
+statistic over 8 samples can have near-zero variance), so the float32 CPU oracle
+itself sits 1e-3 ... 1e-1 from float64 in the early layers: the bound is what "as
+close as a numpy fp32 executor" means for this network.  The distances are
+recorded per tensor (tests/parity.py).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import models as OM
+import parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(got, ref):
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    diff = np.asarray(got, dtype=np.float64).ravel() - ref
+    return float(np.sqrt(np.dot(diff, diff)) / max(1e-30, np.sqrt(np.dot(ref, ref))))
+
+
+_ORACLE = {}
+
+
+def _oracle_step(model, X, y, lr):
+    """float64 and float32 CPU steps, evaluated once for both parametrisations."""
+    if not _ORACLE:
+        net = OM.network("resnet50", bn_mode="pre_activation", image=224)
+        p64 = {v.name: val.astype(np.float64) for v, val in model.variables.items()}
+        p32 = {v.name: val for v, val in model.variables.items()}
+        _ORACLE["f64"] = OM.train_step(net, p64, X.astype(np.float64), y.astype(np.float64), lr)[:3]
+        _ORACLE["f32"] = OM.train_step(net, p32, X, y, lr)[:3]
+    return _ORACLE["f64"], _ORACLE["f32"]
+
+
+@pytest.mark.parametrize("winograd", ["planner", "4"])
+def test_resnet50_full_width_step_matches_oracle(monkeypatch, winograd):
+    from tinyflow_amd import _base, models
+    from tinyflow_amd import autodiff as ad
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    if winograd != "planner":
+        monkeypatch.setenv("TINYFLOW_WINOGRAD", winograd)
+    lr = 0.01
+    model, X, y = models.build("resnet50", batch=8)
+    assert X.shape == (8, 3, 224, 224) and model.variables[model.variable_by_name()["s5b2_c3_W"]].shape == (2048, 512, 1, 1)
+    ex = TrainExecutor(model.loss, lr)
+    ex.init_Variable(dict(model.variables))
+    out = ex.run({model.X: X, model.y_: y})
+    loss = out[0].asnumpy()
+
+    # which 3x3 convolutions run in a Winograd form under this setting
+    forms = []
+    for node in ex.topo_order:
+        if isinstance(node.op, ad.Convolution2DForwardOp) and getattr(node, "cudnnlist", None):
+            buf = ctypes.create_string_buffer(256)
+            for which in range(3):
+                assert _base._LIB.DLGpuConvolutionDescribeKernel(node.cudnnlist[0], which, buf, 256, None) == 0
+                forms.append(buf.value.decode())
+    n_wino = sum("winograd" in f for f in forms)
+    if winograd == "4":
+        assert n_wino >= 3 * 16 - 1, "expected every 3x3 convolution in a Winograd form, found %d" % n_wino
+
+    (loss64, grads64, new64), (loss32, grads32, new32) = _oracle_step(model, X, y, lr)
+    np.testing.assert_allclose(loss, loss64, rtol=1e-4)
+    grad_nodes = dict(zip(ex.Variable_node_list, ex.Variable_node_grad_list))
+    worst = 0.0
+    family = "train step resnet50 full width b8 (%s)" % ("planner" if winograd == "planner" else "F(4x4) forced")
+    for var, g in grad_nodes.items():
+        got = ex.value_of(g).asnumpy()
+        cpu_gap = _rel(grads32[var.name], grads64[var.name])
+        err = _rel(got, grads64[var.name])
+        worst = max(worst, err)
+        parity.compare(got, grads64[var.name], grads32[var.name], family + ", gradients", var.name, 3.0,
+                       assert_ratio=False)
+        assert err <= max(5e-2, 3 * cpu_gap), "gradient of %s: relative L2 %.3g, fp32 CPU oracle %.3g" % (
+            var.name, err, cpu_gap)
+    for arr, var in zip(out[1:], model.variables):
+        parity.compare(arr.asnumpy(), new64[var.name], new32[var.name], family + ", updated parameters", var.name,
+                       3.0, assert_ratio=False)
+        # the update itself (new - old = -lr * gradient) in the gradient's norm and bound
+        old = model.variables[var].astype(np.float64)
+        bound = max(5e-2, 3 * _rel(grads32[var.name], grads64[var.name]))
+        assert _rel(arr.asnumpy().astype(np.float64) - old, new64[var.name] - old) <= bound + 1e-3, var.name
+    print("winograd=%s: %d of %d conv launches in a Winograd form, loss %.6f (oracle %.6f), worst gradient "
+          "relative L2 %.2e" % (winograd, n_wino, len(forms), float(loss[0]), float(loss64[0]), worst))
+    ex.close()

@@ -26,6 +26,18 @@ import numpy as np
 import pytest
 
 from oracle import models as OM
+import parity
+
+# Largest allowed ratio of the HIP error to the fp32 CPU oracle's error (both against the
+# float64 oracle) for each gradient and each updated parameter of a step.  The oracle's
+# fp32 convolutions are numpy matmuls, i.e. BLAS, which spreads every reduction over
+# 16-32 SIMD partial sums; a contraction with one fp32 accumulator per output element
+# rounds along a 16-32 times longer chain, so conv-dominated networks get the larger
+# factor (tests/test_gpu_conv_fullsize.py holds the same kernels to 3x a one-accumulator
+# fp32 loop).
+K_STEP = 3.0
+K_STEP_CONV_STACK = 16.0
+K_STEP_CONV_STACK_WINOGRAD = 32.0
 
 pytestmark = pytest.mark.gpu
 
@@ -42,7 +54,7 @@ def _rel_err(got, ref):
     return float(np.sqrt(np.dot(diff, diff)) / max(1e-30, np.sqrt(np.dot(ref, ref))))
 
 
-def _run_steps(config, lr, steps, build_kw, oracle_kw, calibrated=False):
+def _run_steps(config, lr, steps, build_kw, oracle_kw, calibrated=False, k=K_STEP):
     from tinyflow_amd import models
     from tinyflow_amd.TrainExecute import TrainExecutor
     model, X, y = models.build(config, **build_kw)
@@ -53,14 +65,25 @@ def _run_steps(config, lr, steps, build_kw, oracle_kw, calibrated=False):
     net = OM.network(config, **oracle_kw)
     grad_nodes = dict(zip(ex.Variable_node_list, ex.Variable_node_grad_list))
     X64, y64 = X.astype(np.float64), y.astype(np.float64)
+    traj32 = {v.name: val.astype(np.float32) for v, val in model.variables.items()}   # the fp32 CPU run's own trajectory
     for step in range(steps):
         out = ex.run({model.X: X, model.y_: y})
         got_grads = {var.name: ex.value_of(g).asnumpy() for var, g in grad_nodes.items()}
         got_params = {name: arr.asnumpy() for name, arr in zip(names, out[1:1 + len(names)])}
-        if calibrated:
-            params32 = {k: v.astype(np.float32) for k, v in params.items()}
-            loss32, grads32, _, _ = OM.train_step(net, params32, X, y, lr)
+        # the same step on the CPU in float32: what a numpy fp32 executor produces
+        # (it continues from its own parameters, as the GPU run does, unless both restart
+        # from the GPU's parameters every step in the calibrated comparison)
+        params32 = {k: v.astype(np.float32) for k, v in params.items()} if calibrated else traj32
+        with np.errstate(divide="ignore", invalid="ignore"):   # its loss may overflow to -log(0); only gradients are used
+            loss32, grads32, new32, _ = OM.train_step(net, params32, X, y, lr)
+        traj32 = new32
         loss_ref, grads_ref, params, _ = OM.train_step(net, params, X64, y64, lr)
+        family = "train step %s%s" % (config, " (reduced)" if build_kw else "")
+        for name in names:
+            parity.compare(got_grads[name], grads_ref[name], grads32[name], family + ", gradients",
+                           "%s step %d grad %s" % (config, step, name), k, assert_ratio=not calibrated)
+            parity.compare(got_params[name], params[name], new32[name], family + ", updated parameters",
+                           "%s step %d param %s" % (config, step, name), k, assert_ratio=not calibrated)
         if not calibrated:
             _close(out[0].asnumpy(), loss_ref, "%s step %d loss" % (config, step), rtol=1e-4)
             for name in names:
@@ -88,7 +111,7 @@ def test_lenet5_config2_full_size():
 
 
 def test_vgg16_reduced():
-    _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {})
+    _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {}, k=K_STEP_CONV_STACK)
 
 
 @pytest.mark.parametrize("bn_mode", ["pre_activation", "spatial"])
@@ -111,7 +134,8 @@ def test_train_step_with_winograd_convolutions(monkeypatch, config, force):
     the calibrated comparison above."""
     monkeypatch.setenv("TINYFLOW_WINOGRAD", force)
     if config == "vgg16":
-        _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {})
+        _run_steps("vgg16", 0.01, 2, dict(batch=2, image=32, n_class=10, fc_width=64), {},
+                   k=K_STEP_CONV_STACK_WINOGRAD)
     else:
         _resnet_shallow("pre_activation", later_steps_bound=5e-2)
 

@@ -202,7 +202,10 @@ struct Unit<false> {
 };
 
 // x viewed as [N, C, HW]; block (c, chunk) sums images [chunk*ipc, ...) of channel c.
-// FWD: partial = (sum x, sum x^2); BWD: partial = (sum dy, sum dy*xhat).
+// FWD: partial = (sum (x - p), sum (x - p)^2) with the pivot p = the channel's first
+// element (image 0, pixel 0): sums of shifted values lose nothing to cancellation
+// when |mean| is much larger than the standard deviation, where sum x^2 - m*mean^2
+// in fp32 would.  BWD: partial = (sum dy, sum dy*xhat).
 // The (image, pixel) pairs of a chunk are walked as one flat index so that small
 // feature maps (7x7) keep all lanes busy; VEC: 16-byte loads when HW is a multiple
 // of 4.  Lanes accumulate in fp32 (a few hundred terms each), the block and the
@@ -220,6 +223,7 @@ __global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__
   int n1 = n0 + images_per_chunk;
   if (n1 > N) n1 = N;
   const float mean = BWD ? save_mean[c] : 0.f, istd = BWD ? save_istd[c] : 0.f;
+  const float pivot = BWD ? 0.f : x[(int64_t)c * HW];
   constexpr int W = Unit<VEC>::W;
   const uint32_t row_units = (uint32_t)HW / W;                 // div_row divides by this
   const uint32_t total = (uint32_t)(n1 - n0) * row_units;
@@ -237,8 +241,9 @@ __global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__
         a0 += gv[k];
         b0 += gv[k] * ((xv[k] - mean) * istd);
       } else {
-        a0 += xv[k];
-        b0 += xv[k] * xv[k];
+        const float t = xv[k] - pivot;
+        a0 += t;
+        b0 += t * t;
       }
     }
   }
@@ -255,6 +260,7 @@ __global__ __launch_bounds__(kThreads) void bn_sp_partial_kernel(const float *__
 // statistics; backward (sum dy, sum dy*xhat).
 template <bool BWD>
 __global__ __launch_bounds__(kThreads) void bn_sp_finish_kernel(const double *__restrict__ partial,
+                                                               const float *__restrict__ x,
                                                                float *__restrict__ out0, float *__restrict__ out1,
                                                                int N, int C, int HW, int chunks) {
   const int c = blockIdx.x * kThreads + threadIdx.x;
@@ -269,10 +275,10 @@ __global__ __launch_bounds__(kThreads) void bn_sp_finish_kernel(const double *__
     out1[c] = (float)q;
   } else {
     const double m = (double)N * (double)HW;
-    const double mean_d = s / m;
-    double var = q / m - mean_d * mean_d;
+    const double shifted_mean = s / m;  // mean of x - pivot; the variance does not depend on the pivot
+    double var = q / m - shifted_mean * shifted_mean;
     if (var < 0.0) var = 0.0;
-    out0[c] = (float)mean_d;
+    out0[c] = (float)((double)x[(int64_t)c * HW] + shifted_mean);
     out1[c] = (float)(1.0 / sqrt(var + (double)kEps));
   }
 }
@@ -441,8 +447,8 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
       constexpr bool VEC = decltype(vec_c)::value;
       hipLaunchKernelGGL((bn_sp_partial_kernel<false, VEC>), pgrid, dim3(kThreads), 0, s, x, (const float *)nullptr,
                          (const float *)nullptr, (const float *)nullptr, partial, d->N, d->C, d->HW, ipc, div_row);
-      hipLaunchKernelGGL(bn_sp_finish_kernel<false>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, mean,
-                         istd, d->N, d->C, d->HW, real_chunks);
+      hipLaunchKernelGGL(bn_sp_finish_kernel<false>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, x,
+                         mean, istd, d->N, d->C, d->HW, real_chunks);
       hipLaunchKernelGGL((bn_sp_apply_kernel<false, VEC>), agrid, dim3(kThreads), 0, s, x, (const float *)nullptr, y,
                          (const float *)mean, (const float *)istd, (const float *)nullptr, (const float *)nullptr,
                          0.f, div_row, div_c, units);
@@ -531,8 +537,8 @@ static int bn_backward_impl(const DLArrayHandle input, const DLArrayHandle doutp
         constexpr bool VEC = decltype(vec_c)::value;
         hipLaunchKernelGGL((bn_sp_partial_kernel<true, VEC>), pgrid, dim3(kThreads), 0, s, x, dy, mean, istd, partial,
                            d->N, d->C, d->HW, ipc, div_row);
-        hipLaunchKernelGGL(bn_sp_finish_kernel<true>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, sums,
-                           sums + d->C, d->N, d->C, d->HW, real_chunks);
+        hipLaunchKernelGGL(bn_sp_finish_kernel<true>, dim3(cdiv(d->C, kThreads)), dim3(kThreads), 0, s, partial, x,
+                           sums, sums + d->C, d->N, d->C, d->HW, real_chunks);
         hipLaunchKernelGGL((bn_sp_apply_kernel<true, VEC>), agrid, dim3(kThreads), 0, s, x, dy, dx, mean, istd,
                            (const float *)sums, (const float *)(sums + d->C), m, div_row, div_c, units);
       };
