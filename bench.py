@@ -4,13 +4,19 @@ backward + SGD update) of ResNet-50, batch 64, fp32, on one MI355X, synthetic da
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Prints ONE JSON line.  Next to the throughput it carries
-  "roofline":     achieved vs peak for the kernel variant that takes the most GPU
-                  time in the step (an MFMA implicit-GEMM convolution), measured
-                  with HIP events recorded on the compute stream around every
+  "roofline":     achieved vs fp32 MFMA peak for the BACKWARD contraction kernel symbol
+                  (grad-data or grad-filter) that takes the most GPU time in the step,
+                  measured with HIP events recorded on the compute stream around every
                   convolution launch of the timed steps;
+  "roofline_fwd": the same for the dominant forward symbol;
+  "roofline_bwd": all grad-data launches together and all grad-filter launches together
+                  (executed flops / event time, fraction of peak, slowest symbol of each),
+                  and the single op with the most time in the step;
+  "hbm_kernels":  achieved GB/s against 8 TB/s for the bandwidth-bound gradient ops;
   "cpu_baseline": the CPU oracle (numpy restatement of the same step) timed on
                   this machine's host cores on a bounded sample (a smaller batch),
-                  scaled linearly to images/sec.
+                  scaled linearly to images/sec; the HIP step on that same sample is
+                  checked against it.
 Everything here runs on one GPU; --gpus N with N > 1 is refused.
 """
 import argparse
@@ -26,6 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+PASS_NAMES = {0: "forward", 1: "grad-data", 2: "grad-filter"}
 MFMA_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
 HBM_PEAK_GBS = 8000.0
@@ -67,37 +74,42 @@ def stream_handle(stream_cell):
     return ctypes.cast(stream_cell, ctypes.POINTER(ctypes.c_void_p))[0]
 
 
-# HBM bytes per launch (reads + writes) of each convolution kernel symbol in the
-# default workload, averaged over that symbol's launches in one step: rocprofv3
-# FETCH_SIZE and WRITE_SIZE counter runs of this script, scaled by what the same
-# counters read for a 256 MiB copy (x2.000 and x1.000).  The figures and the
-# commands are in profiles/resnet50_b64_train_step_hbm_traffic.txt; they hold for
-# --config resnet50 --batch 64 only and are reported as null otherwise.
-MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Across4<64, 32>>, StoreBatched>": 210391435,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Along4<128, 16>, StoreNCHW>": 140242015,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, Across4<128, 16>, StoreRowMajor>": 131504118,
-    "gemm_kernel<128, 128, 16, Along4<128, 16>, Along4<128, 16>, StoreNCHW>": 127779549,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Across4<64, 32>, StoreRowMajor>": 222997758,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 180019254,
-    "gemm_kernel<64, 128, 16, Batched<Along4<64, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 179452610,
-    "gemm_kernel<64, 128, 16, Along4<64, 16>, Along4<128, 16>, StoreNCHW>": 227002849,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreScatter>": 225359672,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAlong<128, 16, 0>, StoreNCHW>": 235497575,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAlong<64, 32, 0>, StoreNCHW>": 127443020,
-    "gemm_kernel<64, 64, 32, Batched<Along4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207728188,
-    "gemm_kernel<64, 64, 32, Batched<Across4<64, 32>>, Batched<Along4<64, 32>>, StoreBatched>": 207656627,
-    "gemm_kernel<64, 128, 16, Across4<64, 16>, Along4<128, 16>, StoreNCHW>": 206299823,
-    "gemm_kernel<128, 128, 16, Across4<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 288039008,
-    "gemm_kernel<128, 128, 16, Batched<Along4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134844673,
-    "gemm_kernel<128, 128, 16, Batched<Across4<128, 16>>, Batched<Along4<128, 16>>, StoreBatched>": 134751909,
-    "gemm_kernel<128, 128, 16, DyAcross<128, 16>, GatherAcross<128, 16, 0>, StoreRowMajor>": 89372689,
-    "gemm_kernel<64, 64, 32, Along4<64, 32>, Along4<64, 32>, StoreNCHW>": 132705032,
-    "gemm_kernel<64, 128, 16, Batched<Across4<64, 16>>, Batched<Across4<128, 16>>, StoreBatched>": 151099603,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, Along4<64, 32>, StoreNCHW>": 132824043,
-    "gemm_kernel<64, 64, 32, Across4<64, 32>, GatherAcross<64, 32, 0>, StoreRowMajor>": 171230225,
-    "gemm_kernel<64, 64, 32, PlainAlong<64, 32>, GatherAlong<64, 32, 0>, StoreScatter>": 148485080,
-}
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "resnet50_b64_train_step_hbm_traffic.txt")
+
+
+def _normalise_symbol(name):
+    """Kernel symbol with the spacing differences between profiler versions removed."""
+    return name.replace(" >", ">").replace(", ", ",").strip()
+
+
+def measured_traffic_bytes():
+    """{kernel symbol: HBM bytes per launch (reads + writes)} from the committed summary of
+    the two rocprofv3 counter runs of this script (FETCH_SIZE, WRITE_SIZE, each scaled by
+    what the same counter reads for a copy of known size; the summary states the commands
+    and the factors).  It covers --config resnet50 --batch 64 in per-activation mode; a
+    symbol the summary does not list (a kernel changed since the counter run) reads null."""
+    table = {}
+    try:
+        with open(TRAFFIC_SUMMARY) as fh:
+            lines = fh.read().splitlines()
+    except OSError:
+        return table
+    in_table = False
+    for line in lines:
+        if line.startswith("kernel") and "total MiB" in line:
+            in_table = True
+            continue
+        if in_table:
+            parts = line.rsplit(None, 4)
+            if len(parts) != 5:
+                if table:
+                    break
+                continue
+            try:
+                table[_normalise_symbol(parts[0])] = int(float(parts[4]) * (1 << 20))
+            except ValueError:
+                break
+    return table
 
 
 class ConvTimer(object):
@@ -108,7 +120,7 @@ class ConvTimer(object):
 
     def __init__(self, hip, gpu_op, lib):
         self.hip, self.gpu_op, self.lib = hip, gpu_op, lib
-        self.pairs = []     # (variant, flops, e0, e1)
+        self.pairs = []     # (which, kernel symbol, flops, e0, e1)
         self.pool = []
         self.enabled = False
         self._describe_cache = {}
@@ -150,7 +162,7 @@ class ConvTimer(object):
                 self.lib.DLGpuConvolutionTimeNextKernel(None, None)
                 self.pool += [e0, e1]
             else:
-                self.pairs.append((variant, flops, e0, e1))
+                self.pairs.append((which, variant, flops, e0, e1))
             return ret
         return timed
 
@@ -183,11 +195,12 @@ class ConvTimer(object):
         return max(single - bulk, 0.0)
 
     def collect(self, overhead_ms=0.0):
-        """{variant: [launches, total_ms, total_flops]}; call after a device sync."""
+        """{(which, kernel symbol): [launches, total_ms, total_flops]} with which = 0 forward,
+        1 grad-data, 2 grad-filter; call after a device sync."""
         stats = {}
-        for variant, flops, e0, e1 in self.pairs:
+        for which, variant, flops, e0, e1 in self.pairs:
             ms = max(self.hip.elapsed_ms(e0, e1) - overhead_ms, 1e-6)
-            st = stats.setdefault(variant, [0, 0.0, 0.0])
+            st = stats.setdefault((which, variant), [0, 0.0, 0.0])
             st[0] += 1
             st[1] += ms
             st[2] += flops
@@ -250,18 +263,36 @@ class HbmTimer(object):
 
 
 def cpu_baseline(bn_mode, sample_batch, image, repeats):
-    """The oracle's ResNet-50 step on the host cores, on a reduced batch."""
+    """The oracle's ResNet-50 step on the host cores, on a reduced batch, timed; and the
+    same reduced batch through the HIP step, whose loss and gradients are checked against
+    the oracle's (the product is the thing measured, the oracle the checker)."""
     from oracle import models as OM
     from tinyflow_amd import models
+    from tinyflow_amd.TrainExecute import TrainExecutor
     model, X, y = models.build("resnet50", batch=sample_batch, image=image, bn_mode=bn_mode)
     params = {v.name: val for v, val in model.variables.items()}
     net = OM.network("resnet50", bn_mode=bn_mode, image=image)
     times = []
     for _ in range(repeats + 1):
         t0 = time.perf_counter()
-        OM.train_step(net, params, X, y, 0.01)
+        loss_cpu, grads_cpu, _, _ = OM.train_step(net, params, X, y, 0.01)
         times.append(time.perf_counter() - t0)
     best = float(np.median(times[1:]))  # first call warms BLAS and the allocator
+    ex = TrainExecutor(model.loss, 0.01)
+    ex.init_Variable(dict(model.variables))
+    loss_gpu = float(ex.run({model.X: X, model.y_: y})[0].asnumpy()[0])
+    loss_cpu = float(np.asarray(loss_cpu).ravel()[0])
+    if not abs(loss_gpu - loss_cpu) <= 1e-3 * abs(loss_cpu):
+        raise RuntimeError("HIP step and CPU oracle disagree on the batch-%d loss: %r vs %r"
+                           % (sample_batch, loss_gpu, loss_cpu))
+    worst, worst_name = 0.0, ""
+    for var, g in zip(ex.Variable_node_list, ex.Variable_node_grad_list):
+        ref = grads_cpu[var.name].astype(np.float64).ravel()
+        diff = ex.value_of(g).asnumpy().astype(np.float64).ravel() - ref
+        err = float(np.sqrt(np.dot(diff, diff)) / max(1e-30, np.sqrt(np.dot(ref, ref))))
+        if err > worst:
+            worst, worst_name = err, var.name
+    ex.close()
     try:
         from threadpoolctl import threadpool_info
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
@@ -271,8 +302,12 @@ def cpu_baseline(bn_mode, sample_batch, image, repeats):
         "value": sample_batch / best, "unit": "imgs/sec", "cores": threads, "kind": "port",
         "sample": "oracle numpy fp32 ResNet-50 step (fwd+bwd+SGD, bn_mode=%s) at batch %d, image %d; "
                   "median of %d steps after 1 warm-up, %.2f s per step; images/sec = batch / time "
-                  "(os.cpu_count()=%d, affinity=%d)"
-                  % (bn_mode, sample_batch, image, repeats, best, os.cpu_count(), len(os.sched_getaffinity(0))),
+                  "(os.cpu_count()=%d, affinity=%d).  Checked against the HIP step on the same batch: loss %.6f "
+                  "(HIP) vs %.6f (oracle), worst gradient relative L2 distance %.2e (%s; both are fp32 evaluations "
+                  "of a 50-layer batch-normalised stack at batch %d)"
+                  % (bn_mode, sample_batch, image, repeats, best, os.cpu_count(), len(os.sched_getaffinity(0)),
+                     loss_gpu, loss_cpu, worst, worst_name, sample_batch),
+        "hip_loss": loss_gpu, "oracle_loss": loss_cpu, "worst_gradient_rel_l2": worst,
     }
 
 
@@ -425,29 +460,76 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     imgs_per_sec = args.batch * args.steps / wall
 
-    roofline = None
     pair_overhead = timer.pair_overhead_ms(s)
     stats = timer.collect(pair_overhead)
-    if stats:
-        top = max(stats.items(), key=lambda kv: kv[1][1])
-        name, (launches, total_ms, total_flops) = top
+    gpu_step_ms = gpu_ms / args.steps
+    default_workload = ((args.config, args.batch, args.bn_mode) == ("resnet50", 64, "pre_activation")
+                        and not args.mem_limit_gb)
+    traffic = measured_traffic_bytes() if default_workload else {}
+
+    def symbol_roofline(which, name, launches, total_ms, total_flops):
         achieved = total_flops / (total_ms * 1e-3) / 1e12
-        roofline = {
-            "bound": "mfma", "kernel": name, "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
-            "traffic": (MEASURED_TRAFFIC_BYTES.get(name) if (args.config, args.batch, args.bn_mode) ==
-                        ("resnet50", 64, "pre_activation") and not args.mem_limit_gb else None),
+        return {
+            "bound": "mfma", "pass": PASS_NAMES[which], "kernel": name, "achieved": achieved,
+            "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
+            "traffic": traffic.get(_normalise_symbol(name)),
             "flops_per_launch": total_flops / launches,
             "launches": launches, "avg_launch_ms": total_ms / launches,
-            "share_of_step": total_ms / event_steps / (gpu_ms / args.steps), "steps_with_events": event_steps,
+            "share_of_step": total_ms / event_steps / gpu_step_ms, "steps_with_events": event_steps,
             "event_pair_overhead_us": pair_overhead * 1e3,
         }
+
+    def dominant(passes):
+        """Contraction kernel symbol with the most event time among the given passes."""
+        rows = [(k, v) for k, v in stats.items() if k[0] in passes]
+        if not rows:
+            return None
+        (which, name), (launches, total_ms, total_flops) = max(rows, key=lambda kv: kv[1][1])
+        return symbol_roofline(which, name, launches, total_ms, total_flops)
+
+    def whole_pass(which):
+        """All contraction launches of one pass together, and its slowest symbol."""
+        rows = [(k[1], v) for k, v in stats.items() if k[0] == which]
+        if not rows:
+            return None
+        ms = sum(v[1] for _, v in rows)
+        flops = sum(v[2] for _, v in rows)
+        slow_name, slow = min(rows, key=lambda kv: kv[1][2] / kv[1][1])
+        return {
+            "executed_tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
+            "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "ms_per_step": ms / event_steps,
+            "launches_per_step": sum(v[0] for _, v in rows) / event_steps, "symbols": len(rows),
+            "slowest_symbol": {"kernel": slow_name, "tflops": slow[2] / (slow[1] * 1e-3) / 1e12,
+                               "frac": slow[2] / (slow[1] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
+                               "ms_per_step": slow[1] / event_steps, "launches_per_step": slow[0] / event_steps},
+        }
+
+    # `roofline`: the backward contraction kernel (grad-data or grad-filter) with the most
+    # time in the step -- the metric asks for the backward kernels; the dominant forward
+    # symbol is reported beside it.
+    roofline = dominant((1, 2)) if stats else None
+    roofline_fwd = dominant((0,)) if stats else None
+    roofline_bwd = None
+    if stats:
+        roofline_bwd = {"grad_data": whole_pass(1), "grad_filter": whole_pass(2), "forward": whole_pass(0),
+                        "note": "flops are the ones the kernels execute (Winograd products count their own, "
+                                "2.25x or 4x fewer than the direct form); time is the HIP-event time of the "
+                                "contraction kernels alone, without transform and split-sum passes"}
+        # the single op with the most time in the step, whatever bounds it
+        conv_rows = [("%s %s" % (PASS_NAMES[k[0]], k[1]), v[1] / event_steps, "mfma",
+                      v[2] / (v[1] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS) for k, v in stats.items()]
+        hbm_rows = [(h["op"], h["avg_launch_us"] * h["launches"] / 2 * 1e-3, "hbm", h["frac_of_hbm_peak"])
+                    for h in (hbm_kernels or [])]   # the bandwidth-bound ops were timed over two steps
+        if conv_rows or hbm_rows:
+            name, ms, bound, frac = max(conv_rows + hbm_rows, key=lambda r: r[1])
+            roofline_bwd["top_of_step"] = {"op": name, "ms_per_step": ms, "bound": bound, "frac_of_peak": frac,
+                                           "share_of_step": ms / gpu_step_ms}
         if args.breakdown:
             conv_ms = sum(v[1] for v in stats.values()) / event_steps
-            sys.stderr.write("GPU ms/step (events): %.3f, conv kernels: %.3f\n" % (gpu_ms / args.steps, conv_ms))
-            for k, (n, ms, fl) in sorted(stats.items(), key=lambda kv: -kv[1][1]):
-                sys.stderr.write("  %-34s launches/step %5.1f  ms/step %8.3f  TFLOP/s %7.2f\n"
-                                 % (k, n / event_steps, ms / event_steps, fl / (ms * 1e-3) / 1e12))
+            sys.stderr.write("GPU ms/step (events): %.3f, conv kernels: %.3f\n" % (gpu_step_ms, conv_ms))
+            for (which, k), (n, ms, fl) in sorted(stats.items(), key=lambda kv: -kv[1][1]):
+                sys.stderr.write("  %-11s %-90s launches/step %5.1f  ms/step %8.3f  TFLOP/s %7.2f\n"
+                                 % (PASS_NAMES[which], k, n / event_steps, ms / event_steps, fl / (ms * 1e-3) / 1e12))
 
     result = {
         "metric": "train imgs/sec ResNet-50 b64 fp32 fwd+bwd; bwd kernel % of HBM/MFMA peak",
@@ -461,6 +543,8 @@ def main():
         "host_fed": {"ms_per_step": host_fed_ms, "imgs_per_sec": args.batch * 1e3 / host_fed_ms, "steps": host_steps,
                      "note": "batch re-uploaded from pageable host memory every step (PCIe-inclusive)"},
         "roofline": roofline,
+        "roofline_fwd": roofline_fwd,
+        "roofline_bwd": roofline_bwd,
         "hbm_kernels": hbm_kernels,
         "fused_bn_relu": fused,
     }
@@ -483,7 +567,7 @@ def main():
         }
         ex.close()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(args.bn_mode, args.cpu_batch, 224, 2)
+        result["cpu_baseline"] = cpu_baseline(args.bn_mode, args.cpu_batch, 224, 3)
     print(json.dumps(result))
 
 
