@@ -239,6 +239,52 @@ def test_conv_adjoint_identities_full_size(rt, layer):
     np.testing.assert_allclose(y[:1, k_some], y_ref, rtol=1e-3, atol=1e-5 * scale)
 
 
+# Layers whose launches fold tiles in the kernel: a short k-split whose pieces are added by
+# the last workgroup of each tile (forward of 1024 -> 256 at 14x14), and a remainder
+# round cut into pieces (forward and grad-data of 512 -> 1024 stride 2, 784 tiles on 256 CUs).
+FOLDED_LAYERS = [(64, 1024, 14, 256, 1, 1), (64, 512, 28, 1024, 1, 2), (64, 256, 14, 1024, 1, 1),
+                 (64, 512, 7, 2048, 1, 1)]
+
+
+@pytest.mark.parametrize("layer", FOLDED_LAYERS, ids=lambda l: "x".join(str(v) for v in l))
+def test_in_kernel_fold_matches_the_unfolded_launch(rt, monkeypatch, layer):
+    """Tiles computed in pieces and added by the last workgroup to arrive must equal the
+    same launch without pieces (up to the rounding of a different summation order), on
+    every element and on every one of many repetitions: a piece read before it was
+    complete, or from a stale cache line, would show as a wrong 64x64 or 128x128 block.
+    Repetitions of the folded launch must also agree with each other bit for bit."""
+    from tinyflow_amd import gpu_op, ndarray
+    N, C, HW, K, R, stride = layer
+    rng = np.random.RandomState(parity.stable_seed(layer))
+    x = rng.normal(0, 1, (N, C, HW, HW)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(2.0 / (C * R * R)), (K, C, R, R)).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", "VALID", stride, stride)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
+
+    def run():
+        gy, gdx, gdw = ndarray.empty(out_shape, rt.ctx), ndarray.empty(x.shape, rt.ctx), ndarray.empty(w.shape, rt.ctx)
+        for arr in (gy, gdx, gdw):
+            gpu_op.array_set(arr, np.nan, rt.stream)
+        assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+        assert gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream) == 0
+        assert gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream) == 0
+        return gy.asnumpy(), gdx.asnumpy(), gdw.asnumpy()
+
+    monkeypatch.setenv("TINYFLOW_FOLD", "0")
+    plain = run()
+    monkeypatch.setenv("TINYFLOW_FOLD", "3")
+    first = run()
+    assert any(not np.array_equal(a, b) for a, b in zip(plain, first)), "no launch of this layer folds anything"
+    for a, b, what in zip(plain, first, ("forward", "grad-data", "grad-filter")):
+        scale = max(1.0, float(np.abs(a).max()))
+        np.testing.assert_allclose(b, a, rtol=1e-4, atol=1e-5 * scale, err_msg=what)
+    for _ in range(15):
+        again = run()
+        for a, b in zip(first, again):
+            assert a.tobytes() == b.tobytes()
+
+
 def test_conv_rejects_mismatched_arrays(rt, capfd):
     from tinyflow_amd import gpu_op, ndarray
     out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape((2, 3, 8, 8), (4, 3, 3, 3), "NCHW", "SAME", 1, 1)

@@ -19,6 +19,7 @@
 // in memory for NCHW/KCRS, so global loads and stores coalesce without any
 // layout change of the activations.
 #include "gemm_core.h"
+#include "gemm_launch.h"
 #include "internal.h"
 
 #include <algorithm>
@@ -744,7 +745,7 @@ template <int BM, int BN, int BK, class AL, class BL, class EP>
 void launch(const AL &al, const BL &bl, const EP &ep, int K, const Geometry &g, hipStream_t s, int batch = 1) {
   if (next_kernel_start) (void)hipEventRecord(next_kernel_start, s);
   hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, EP>), dim3(g.blocks(), batch), dim3(THREADS), 0, s, al, bl, ep,
-                     K, g.k_per_split, g.tiles_m, g.tiles_n);
+                     K, g.k_per_split, g.tiles_m, g.tiles_n, g.fold());
   if (next_kernel_stop) (void)hipEventRecord(next_kernel_stop, s);
   next_kernel_start = next_kernel_stop = nullptr;
 }
@@ -1318,7 +1319,13 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
     return finish(s, "DLGpuConvolution2DForward");
   }
   const int bm = plan.bm, bn = plan.bn;
-  const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+  Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+  plan_fold(g, K, stage_depth(bm, bn), 1);
+  FoldBuffers fb;
+  if (const int rc = acquire_fold(g, bm, bn, 1, s, fb)) {
+    if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);
+    return rc == 1 ? 0 : -1;
+  }
   float *partial = nullptr;
   if (g.splits > 1) {
     const size_t bytes = (size_t)g.splits * numel(output) * sizeof(float);
@@ -1365,6 +1372,7 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
     launch_split_sum(partial, (float *)output->data, numel(output), g.splits, s);
     device_free(partial);
   }
+  release_fold(fb);
   return finish(s, "DLGpuConvolution2DForward");
 }
 
@@ -1406,12 +1414,24 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   }
   const uint32_t w_bytes = (uint32_t)(numel(filter) * 4), dy_bytes = (uint32_t)(numel(doutput) * 4);
   const int PQ = d->P * d->Q;
+  // a strided filter larger than 1x1 always runs on the small tile, unsplit
+  const bool strided_taps = RS > 1 && !(d->u == 1 && d->v == 1);
+  const int g_bm = strided_taps ? 64 : plan.bm, g_bn = strided_taps ? 64 : plan.bn;
+  Geometry g = make_geometry(M, plan.N, K, g_bm, g_bn, strided_taps ? 1 : plan.splits, stage_depth(g_bm, g_bn));
+  plan_fold(g, K, stage_depth(g_bm, g_bn), 1);
+  FoldBuffers fb;
+  if (const int rc = acquire_fold(g, g_bm, g_bn, 1, s, fb)) {
+    if (wt_scratch) device_free(wt_scratch);
+    if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);
+    return rc == 1 ? 0 : -1;
+  }
   float *partial = nullptr;
-  if (plan.splits > 1) {
-    const size_t bytes = (size_t)plan.splits * numel(dinput) * sizeof(float);
+  if (g.splits > 1) {
+    const size_t bytes = (size_t)g.splits * numel(dinput) * sizeof(float);
     partial = (float *)device_alloc(bytes);
     if (!partial) {
       if (wt_scratch) device_free(wt_scratch);
+      release_fold(fb);
       if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
@@ -1426,7 +1446,6 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     // 1x1 filter (pad 0): compact GEMM over the output pixels + scatter
     const int N = plan.N;
     const int bm = plan.bm, bn = plan.bn;
-    const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
     with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
       constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
       auto with_epilogue = [&](const auto &al, const auto &bl) {
@@ -1458,7 +1477,6 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     const int bm = plan.bm, bn = plan.bn;
     StoreNCHW ep{dst, M, N, FastDiv((uint32_t)HW), HW, dx_count};
     if (d->u == 1 && d->v == 1) {
-      const Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
       with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
         constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
         GatherAlong<BN, BK, 1> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv((uint32_t)RS),
@@ -1470,7 +1488,6 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
       });
     } else {
       // strided filter larger than 1x1: every input pixel, taps filtered by divisibility
-      const Geometry g = make_geometry(M, N, K, 64, 64, 1, 32);
       PlainAlong<64, 32> al{wt, w_bytes, d->C, M, K};
       GatherAlong<64, 32, 2> bl{(const float *)doutput->data, dy_bytes, K, N, FastDiv((uint32_t)RS),
                             FastDiv((uint32_t)d->S), PQ,
@@ -1481,9 +1498,10 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     }
   }
   if (partial) {
-    launch_split_sum(partial, (float *)dinput->data, dx_count, plan.splits, s);
+    launch_split_sum(partial, (float *)dinput->data, dx_count, g.splits, s);
     device_free(partial);
   }
+  release_fold(fb);
   if (wt_scratch) device_free(wt_scratch);
   return finish(s, "DLGpuConvolutionBackwardData");
 }
@@ -1511,12 +1529,19 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
 
   const int bm = plan.bm, bn = plan.bn;
   Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
+  plan_fold(g, K, stage_depth(bm, bn), 1);
+  FoldBuffers fb;
+  if (const int rc = acquire_fold(g, bm, bn, 1, s, fb)) {
+    if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);
+    return rc == 1 ? 0 : -1;
+  }
   float *dst = (float *)dfilter->data;
   float *partial = nullptr;
   if (g.splits > 1) {
     const size_t bytes = (size_t)g.splits * M * N * sizeof(float);
     partial = (float *)device_alloc(bytes);
     if (!partial) {
+      release_fold(fb);
       if (memorytoSaving) *memorytoSaving = shortfall(bytes);
       return 0;
     }
@@ -1560,5 +1585,6 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
     launch_split_sum(partial, (float *)dfilter->data, (int64_t)M * N, g.splits, s);
     device_free(partial);
   }
+  release_fold(fb);
   return finish(s, "DLGpuConvolutionBackwardFilter");
 }

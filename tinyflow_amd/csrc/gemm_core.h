@@ -306,8 +306,39 @@ struct StoreRowMajor {
   }
 };
 
+// ---- in-kernel fold of k-split tiles ---------------------------------------------------
+// Some output tiles of a launch can be computed by several workgroups ("pieces"),
+// each over its own range of the reduction, without a second pass: a piece
+// writes its raw accumulators to scratch, takes a ticket for its tile, and the
+// piece that draws the last ticket adds all pieces of the tile in piece order
+// (its own included, re-read from scratch) and runs the epilogue.  The order of
+// the additions is fixed, so the result does not depend on which piece arrives
+// last.  Nobody waits for anybody: a piece that is not last simply exits.
+// Used in two ways by the hosts:
+//   * every tile folded (first_tile = 0): a k-split of a few pieces without the
+//     separate sum pass;
+//   * only the tiles past the last full round over the CUs folded: the remainder
+//     round, which would keep a fraction of the CUs busy for a whole tile time,
+//     becomes about one short piece per CU.
+struct Fold {
+  float *scratch;      // [batch][folded tile][piece][BM * BN] accumulators, lane-major
+  unsigned *tickets;   // [batch][folded tile], zero before the launch; the last piece zeroes its counter again
+  int first_tile;      // tiles [0, first_tile) are plain, tiles [first_tile, tiles) are folded
+  int plain_blocks;    // workgroups of the plain tiles (first_tile * plain splits); they come first in the grid
+  int pieces;          // workgroups per folded tile; 0 or 1: nothing is folded
+  int k_per_piece;     // reduction steps per piece (a multiple of BK)
+};
+
+// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; this gives
+// each XCD a contiguous range of the n logical ids instead.
+__device__ inline int xcd_contiguous(int id, int n) {
+  const int per_xcd = n >> 3;
+  return id < (per_xcd << 3) ? (id & 7) * per_xcd + (id >> 3) : id;
+}
+
 // ---- the kernel ----------------------------------------------------------------------
-// Work decomposition: gridDim.x = tiles_m * tiles_n * splits.  Hardware hands
+// Work decomposition: gridDim.x = tiles_m * tiles_n * splits (plus, with a fold, the
+// pieces of the folded tiles behind the plain workgroups).  Hardware hands
 // consecutive workgroup ids to the 8 XCDs round-robin; the remap below gives
 // each XCD a contiguous range of logical tile ids, ordered m-fastest, so the
 // workgroups that share one B tile (the large, gathered operand) also share an
@@ -315,7 +346,8 @@ struct StoreRowMajor {
 // epilogue; there is no data-dependent loop.
 template <int BM, int BN, int BK, class ALoader, class BLoader, class Epilogue>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const BLoader bl, const Epilogue ep,
-                                                      int k_extent, int k_per_split, int tiles_m, int tiles_n) {
+                                                      int k_extent, int k_per_split, int tiles_m, int tiles_n,
+                                                      const Fold fold) {
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   static_assert(TM >= 1 && TN >= 1, "tile too small for a 2x2 wave grid");
@@ -328,19 +360,31 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
 
-  // XCD-aware logical id
-  const int nb = gridDim.x;
-  const int per_xcd = nb >> 3;
-  int logical = blockIdx.x;
-  if (logical < (per_xcd << 3)) logical = (logical & 7) * per_xcd + (logical >> 3);
-  const int tm = logical % tiles_m;
-  const int rest = logical / tiles_m;
-  const int tn = rest % tiles_n;
-  const int split = rest / tiles_n;
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int k_begin = split * k_per_split;
-  int k_end = k_begin + k_per_split;
+  // which tile, and which part of the reduction (all of this is scalar arithmetic)
+  const int tiles = tiles_m * tiles_n;
+  const bool folding = fold.pieces > 1;
+  const bool folded = folding && (int)blockIdx.x >= fold.plain_blocks;
+  int tile, split, k_begin, k_end, fold_tile = 0, piece = 0;
+  if (!folded) {
+    const int plain_tiles = folding ? fold.first_tile : tiles;
+    const int logical = xcd_contiguous((int)blockIdx.x, folding ? fold.plain_blocks : (int)gridDim.x);
+    tile = logical % plain_tiles;
+    split = logical / plain_tiles;
+    k_begin = split * k_per_split;
+    k_end = k_begin + k_per_split;
+  } else {
+    const int fold_tiles = tiles - fold.first_tile;
+    const int logical = xcd_contiguous((int)blockIdx.x - fold.plain_blocks, (int)gridDim.x - fold.plain_blocks);
+    fold_tile = logical % fold_tiles;
+    piece = logical / fold_tiles;
+    tile = fold.first_tile + fold_tile;
+    split = 0;
+    k_begin = piece * fold.k_per_piece;
+    k_end = k_begin + fold.k_per_piece;
+  }
   if (k_end > k_extent) k_end = k_extent;
+  const int tm = tile % tiles_m, tn = tile / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
 
   typename ALoader::State sa;
   typename BLoader::State sb;
@@ -411,6 +455,72 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
     buf ^= 1;
   }
 
+  if (folded) {  // uniform over the workgroup
+    // The pieces travel through scratch with device-scope ("sc1") stores and loads:
+    // such an access is coherent across the XCDs' L2s by itself, so no cache-wide
+    // write-back or invalidate is needed (a __threadfence() here costs exactly that
+    // and slows every workgroup of the XCD down).  Ordering: all stores of the piece
+    // have been acknowledged (s_waitcnt 0) before the barrier that precedes the ticket.
+    constexpr int SC1 = 16;  // device scope in the cache-policy operand of the buffer instructions
+    __shared__ unsigned is_last;
+    const int fold_tiles = tiles - fold.first_tile;
+    const size_t slot = (size_t)blockIdx.y * fold_tiles + fold_tile;
+    constexpr uint32_t kPieceBytes = (uint32_t)(BM * BN) * 4u;
+    const __amdgpu_buffer_rsrc_t pieces_of_tile =
+        make_rsrc(fold.scratch + slot * fold.pieces * (size_t)(BM * BN), (uint32_t)fold.pieces * kPieceBytes);
+    const uint32_t lane_off = (uint32_t)tid * 16u;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(
+              __builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), pieces_of_tile,
+              (int)((uint32_t)piece * kPieceBytes + (uint32_t)((i * TN + j) * 4 + q) * (THREADS * 16u) + lane_off), 0,
+              SC1);
+        }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) is_last = atomicAdd(fold.tickets + slot, 1u) == (unsigned)(fold.pieces - 1);
+    __syncthreads();
+    if (!is_last) return;
+    // Last piece of the tile: add the pieces in piece order, four accumulator
+    // registers at a time (the sums go straight to the epilogue, so the fold needs
+    // no registers beyond the loads in flight), and clear the ticket.
+    typename Epilogue::State sf;
+    ep.template init<TN>(sf, n0 + wn * WN, lane, 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        f32x4v sum[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sum[q] = f32x4v{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < fold.pieces; ++p) {
+          f32x4v part[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            part[q] = __builtin_bit_cast(
+                f32x4v, __builtin_amdgcn_raw_buffer_load_b128(
+                            pieces_of_tile,
+                            (int)((uint32_t)p * kPieceBytes + (uint32_t)((i * TN + j) * 4 + q) * (THREADS * 16u) + lane_off),
+                            0, SC1));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sum[q] += part[q];
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * lrow + (v & 3);
+          const int n = n0 + wn * WN + 32 * j + lcol;
+          ep.store(sf, m, n, j, sum[v >> 2][v & 3]);
+        }
+      }
+    if (tid == 0) fold.tickets[slot] = 0u;  // ready for the next launch on this stream
+    return;
+  }
+
   typename Epilogue::State se;
   ep.template init<TN>(se, n0 + wn * WN, lane, split);
 #pragma unroll
@@ -428,7 +538,22 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
 // Host-side launch geometry shared by the users.
 struct Geometry {
   int tiles_m, tiles_n, splits, k_per_split;
-  unsigned blocks() const { return (unsigned)(tiles_m * tiles_n * splits); }
+  // in-kernel fold (see Fold): tiles from fold_first_tile on are computed by fold_pieces
+  // workgroups each; fold_pieces <= 1: none
+  int fold_first_tile = 0, fold_pieces = 0, fold_k_per_piece = 0;
+  int tiles() const { return tiles_m * tiles_n; }
+  int folded_tiles() const { return fold_pieces > 1 ? tiles() - fold_first_tile : 0; }
+  int plain_blocks() const { return (fold_pieces > 1 ? fold_first_tile : tiles()) * splits; }
+  unsigned blocks() const { return (unsigned)(plain_blocks() + folded_tiles() * fold_pieces); }
+  size_t fold_scratch_bytes(int bm, int bn, int batch = 1) const {
+    return (size_t)batch * folded_tiles() * fold_pieces * bm * bn * sizeof(float);
+  }
+  float *fold_scratch = nullptr;        // set by the host once the buffers are there
+  unsigned *fold_ticket_words = nullptr;
+  Fold fold() const {
+    if (fold_pieces <= 1) return Fold{nullptr, nullptr, 0, 0, 0, 0};
+    return Fold{fold_scratch, fold_ticket_words, fold_first_tile, plain_blocks(), fold_pieces, fold_k_per_piece};
+  }
 };
 inline Geometry make_geometry(int M, int N, int K, int bm, int bn, int splits, int BK = 32) {
   Geometry g;

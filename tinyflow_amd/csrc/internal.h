@@ -25,6 +25,10 @@ hipStream_t stream_of(void **cell);      // cell written by DLGpuCreatecudaStrea
 bool sync_every_op();                    // TINYFLOW_SYNC_EVERY_OP=1
 int finish(hipStream_t s, const char *what);  // launch-error check (+ optional sync)
 
+// Zeroed counters for the in-kernel fold of the contraction kernels, one set per stream.
+constexpr int kFoldTicketSlots = 4096;
+unsigned *fold_tickets(hipStream_t s);
+
 // ---- small host utilities -----------------------------------------------------
 inline int64_t numel(const DLArray *a) {
   int64_t n = 1;

@@ -10,6 +10,7 @@
 // connected layer) are split along k into partial products that a second,
 // fixed-order pass adds up, so results do not depend on scheduling.
 #include "gemm_core.h"
+#include "gemm_launch.h"
 #include "internal.h"
 
 using namespace tf;
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(256) void split_sum_vec_kernel(const f32x4 *__restr
 template <int BM, int BN, int BK, class AL, class BL>
 void launch(const AL &al, const BL &bl, const StoreRowMajor &ep, int K, const Geometry &g, hipStream_t s) {
   hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, AL, BL, StoreRowMajor>), dim3(g.blocks()), dim3(THREADS), 0, s,
-                     al, bl, ep, K, g.k_per_split, g.tiles_m, g.tiles_n);
+                     al, bl, ep, K, g.k_per_split, g.tiles_m, g.tiles_n, g.fold());
 }
 
 template <int BM, int BN, int BK>
@@ -184,6 +185,12 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   const int tiles = cdiv(M, bm) * cdiv(N, bn);
   const int splits = choose_splits(tiles, (int)K, 256);
   Geometry g = make_geometry((int)M, (int)N, (int)K, bm, bn, splits);
+  plan_fold(g, (int)K, big ? 16 : 32, 1);
+  FoldBuffers fb;
+  if (acquire_fold(g, bm, bn, 1, s, fb) != 0) {  // no scratch (this entry point cannot report it): no fold
+    release_fold(fb);
+    g = make_geometry((int)M, (int)N, (int)K, bm, bn, splits);
+  }
 
   float *dst = (float *)matC->data;
   float *partial = nullptr;
@@ -206,5 +213,6 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
     launch_split_sum(partial, (float *)matC->data, M * N, g.splits, s);
     device_free(partial);
   }
+  release_fold(fb);
   return finish(s, "DLGpuMatrixMultiply");
 }

@@ -23,7 +23,13 @@ struct StreamRec {
   hipStream_t stream;
   hipEvent_t event;   // reusable marker for cross-stream ordering
   bool runs_kernels;  // an op entry point has launched on it (copy-only streams stay false)
+  unsigned *fold_tickets = nullptr;  // counters of the contraction kernels' in-kernel fold (see fold_tickets)
 };
+
+__global__ void zero_words_kernel(unsigned *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
 
 struct Runtime {
   std::mutex mu;
@@ -391,6 +397,33 @@ hipStream_t stream_of(void **cell) {
   return s;
 }
 
+// Ticket counters for the contraction kernels that fold k-split tiles in the kernel
+// itself: kFoldTicketSlots words per stream, zero between launches (the kernels
+// restore the zeros; launches on one stream run one after the other, so they can
+// share the words).  Allocated on first use and cleared by a fill kernel on `s`.
+unsigned *fold_tickets(hipStream_t s) {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  static unsigned *default_stream_tickets = nullptr;
+  unsigned **cell = &default_stream_tickets;
+  for (auto &rec : r.streams)
+    if (rec.stream == s) {
+      cell = &rec.fold_tickets;
+      break;
+    }
+  if (!*cell) {
+    void *p = nullptr;
+    if (hipMalloc(&p, kFoldTicketSlots * sizeof(unsigned)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(kFoldTicketSlots, 256)), dim3(256), 0, s, (unsigned *)p,
+                       kFoldTicketSlots);
+    *cell = (unsigned *)p;
+  }
+  return *cell;
+}
+
 bool sync_every_op() {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
@@ -650,7 +683,7 @@ extern "C" int DLGpuCreatecudaStream(void **cell) {
     Runtime &r = rt();
     std::lock_guard<std::mutex> g(r.mu);
     r.init();
-    r.streams.push_back({s, ev, false});
+    r.streams.push_back({s, ev, false, nullptr});
   }
   *cell = s;
   return 0;
@@ -667,6 +700,7 @@ extern "C" int DLGpuDestroycudaStream(void **cell) {
     for (size_t i = 0; i < r.streams.size(); ++i)
       if (r.streams[i].stream == s) {
         ev = r.streams[i].event;
+        if (r.streams[i].fold_tickets) (void)hipFree(r.streams[i].fold_tickets);  // waits for the device
         r.streams.erase(r.streams.begin() + i);
         found = true;
         break;
