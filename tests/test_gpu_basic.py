@@ -344,11 +344,29 @@ def test_fused_multi_tensor_sgd_and_adam(rt):
     bit (same arithmetic per element; Adam: same expressions as the two-kernel form)."""
     from tinyflow_amd import gpu_op
     rng = np.random.RandomState(32)
-    shapes = [(64, 3, 3, 3), (10,), (1,), (129, 7), (2, 2)]
+    _fused_case(rt, scattered=False)
+
+
+def test_fused_multi_tensor_updates_with_scattered_indices(rt):
+    """The same with the index tables in a shuffled order: no runs of consecutive offsets,
+    so the launch walks the per-parameter tables instead of whole pieces of tensors."""
+    _fused_case(rt, scattered=True)
+
+
+def _fused_case(rt, scattered):
+    from tinyflow_amd import gpu_op
+    # several pieces per tensor (a piece is 4096 elements), odd sizes, one-element tensors
+    shapes = [(64, 3, 3, 3), (10,), (1,), (129, 7), (2, 2), (5000, 3), (4096,), (3, 4099)]
     sizes = [int(np.prod(s)) for s in shapes]
     number, offset = _flat_index_tables(sizes)
     count = len(number)
-    tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, count)
+    if scattered:
+        order = np.random.RandomState(31).permutation(count)
+        number, offset = [number[i] for i in order], [offset[i] for i in order]
+        tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, count)
+    else:   # numpy tables, as the step executor passes them
+        tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(np.array(number, np.int32), np.array(offset, np.int64),
+                                                                 count)
 
     def fresh():
         r = np.random.RandomState(33)

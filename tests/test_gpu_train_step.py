@@ -214,6 +214,32 @@ def test_fused_bn_relu_executor_is_bit_identical():
             assert a.tobytes() == b.tobytes()
 
 
+@pytest.mark.gpu
+def test_fused_update_is_bit_identical_to_per_variable_updates():
+    """TrainExecutor(fused_update=True) applies every SGD update of the step with one
+    multi-tensor launch behind the last node; losses and parameters over three steps
+    must have the bits of the executor that issues one update node per variable."""
+    from tinyflow_amd import models
+    from tinyflow_amd.TrainExecute import TrainExecutor
+    runs = []
+    for fused in (False, True):
+        rng = np.random.RandomState(22)
+        X, y = models.synthetic_batch(rng, (16, 3, 64, 64), 10, "normal")
+        model = models.resnet(rng, [2, 1, 1, 1], 16, image=64, n_class=10, bn_mode="pre_activation", width=8)
+        ex = TrainExecutor(model.loss, 0.01, fused_update=fused)
+        ex.init_Variable(dict(model.variables))
+        steps = []
+        for _ in range(3):
+            out = ex.run({model.X: X, model.y_: y})
+            steps.append([o.asnumpy() for o in out])
+        assert (ex._fused_sgd is not None) == fused
+        runs.append(steps)
+        ex.close()
+    for a_step, b_step in zip(*runs):
+        for a, b in zip(a_step, b_step):
+            assert a.tobytes() == b.tobytes()
+
+
 @pytest.mark.parametrize("config", ["mlp", "lenet5"])
 def test_adam_executor_matches_oracle(config):
     """Three Adam steps (the reference's TrainExecuteAdam flow): loss, gradients, both

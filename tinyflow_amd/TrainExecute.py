@@ -20,13 +20,21 @@ from . import gpu_op, ndarray
 class TrainExecutor(object):
     """Runs forward + backward + SGD update for one loss node."""
 
-    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), fuse_bn_relu=False):
+    def __init__(self, targetloss, learning_rate, ctx=ndarray.gpu(0), fuse_bn_relu=False, fused_update=True):
         """``fuse_bn_relu`` (no counterpart in the reference): evaluate every batch
         norm whose only reader is a ReLU together with that ReLU, forward and
         backward, through the fused entry points.  Results are bit-identical; the
         batch-norm output and the ReLU's input gradient are then never materialised
-        (``value_of`` does not know them)."""
+        (``value_of`` does not know them).
+
+        ``fused_update``: apply all SGD updates of a step with one call of the
+        multi-tensor entry point (``sgd_compute_o``, reference gpu_op.py:939-945) behind
+        the last node of the step instead of one ``sgd_update`` per variable.  Every
+        update still comes after the last reader of its parameter, which is all
+        ``swapsgd`` asks for, and the arithmetic per element is the same."""
         self.fuse_bn_relu = fuse_bn_relu
+        self.fused_update = fused_update
+        self._fused_sgd = None
         self.fused_pairs = 0
         self.targetloss = targetloss
         self.learning_rate = learning_rate
@@ -75,6 +83,7 @@ class TrainExecutor(object):
         self.infer_shape({node: np.shape(value) for node, value in feed_dict.items()})
         plan = []
         fused = {}
+        fused_sgd = []   # (parameter array, gradient array, learning rate) of the updates applied in one call
         if self.fuse_bn_relu:
             fused.update(find_bn_relu_pairs(self.topo_order, {self.targetloss}))
             fused.update(find_add_relu_pairs(self.topo_order, {self.targetloss}, self.node_to_shape_map))
@@ -98,6 +107,9 @@ class TrainExecutor(object):
                 continue
             assert node.isw not in (1, 2), "no value fed for %s" % node.name
             input_vals = [self.node_to_arr_map[i] for i in node.inputs]
+            if node.issgd and self.fused_update and isinstance(node.op, ad.SgdOp):
+                fused_sgd.append((input_vals[0], input_vals[1], node.learning_rate))
+                continue
             if node.issgd:
                 node_val = None  # updates its parameter in place
             else:
@@ -105,6 +117,8 @@ class TrainExecutor(object):
                 self.node_to_arr_map[node] = node_val
             plan.append((node.op.compute, node, input_vals, node_val))
         self._plan = plan
+        if fused_sgd:
+            self._fused_sgd = _FusedSgd(fused_sgd)
         self.isfirstrun = 1
 
     def run(self, feed_dict, Accuracy_node=None, convert_to_numpy_ret_vals=False):
@@ -121,6 +135,8 @@ class TrainExecutor(object):
             wanted = compute(node, input_vals, node_val, *handles)
             if wanted:
                 raise MemoryError("%s: %d bytes of device scratch could not be allocated" % (node.name, wanted))
+        if self._fused_sgd is not None:
+            self._fused_sgd.apply()
         result = [self.node_to_arr_map[self.targetloss]]
         result += [self.node_to_arr_map[v] for v in reversed(self.Variable_node_list)]
         if Accuracy_node is not None:
@@ -151,6 +167,34 @@ class TrainExecutor(object):
             self.close()
         except Exception:   # interpreter shutdown: the library may already be gone
             pass
+
+
+class _FusedSgd(object):
+    """All SGD updates of a step as one launch: the pointer tables and the index ->
+    (tensor, offset) tables of ``sgd_compute_o`` (reference gpu_op.py:887-945), built
+    once for the step's parameter and gradient arrays, which keep their storage from
+    step to step.  The call has no stream argument: it runs on the default stream,
+    which is ordered behind the executor's stream and in front of its next launch."""
+
+    def __init__(self, updates):
+        rates = set(lr for _, _, lr in updates)
+        assert len(rates) == 1, "one learning rate per step"
+        self.learning_rate = rates.pop()
+        self.arrays = [(w, g) for w, g, _ in updates]   # keeps the storage alive
+        sizes = [int(np.prod(w.shape)) for w, _ in self.arrays]
+        for (w, g), n in zip(self.arrays, sizes):
+            assert int(np.prod(g.shape)) == n, "gradient and parameter sizes differ"
+        self.count = int(sum(sizes))
+        assert self.count < 2 ** 31
+        number = np.repeat(np.arange(len(sizes), dtype=np.int32), sizes)
+        starts = np.cumsum([0] + sizes[:-1])
+        offset = (np.arange(self.count, dtype=np.int64) - np.repeat(starts, sizes)).astype(np.int32)
+        self.tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, self.count)
+        self.pointers = gpu_op.get_n2_cuda_pointer([w.handle.contents.data for w, _ in self.arrays],
+                                                   [g.handle.contents.data for _, g in self.arrays], len(sizes))
+
+    def apply(self):
+        gpu_op.sgd_compute_o(self.pointers, self.tables, self.count, self.learning_rate)
 
 
 def find_bn_relu_pairs(topo_order, outputs):

@@ -14,6 +14,11 @@
 #include "gemm_core.h"
 #include "internal.h"
 
+#include <algorithm>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
 using namespace tf;
 using tf::gemm::FastDiv;
 
@@ -128,6 +133,83 @@ __global__ __launch_bounds__(kThreads) void adam_multi_kernel(float **w, float *
   }
 }
 
+// ---- fused multi-tensor updates, run form -----------------------------------------
+// The per-parameter (tensor number, offset) tables of the fused optimizers describe,
+// in every real use, whole tensors laid end to end: runs of consecutive offsets
+// inside one tensor.  DLGpuGetIndextoVaribaleNumberCudaPointer detects that on the
+// host arrays and records the runs cut into pieces of kRunPiece elements; a launch
+// whose tables were built that way gives one workgroup one piece and streams it like
+// the single-tensor engine (16-byte vectors, 12 bytes per parameter for SGD) instead
+// of reading two 4-byte indices per parameter.  Same arithmetic per element, so the
+// result has the bits of the indexed form.
+constexpr int kRunPiece = kVecPerBlock * 4;  // 4096 elements = 16 KiB per operand
+struct RunPiece {
+  int tensor;   // index into the pointer tables
+  int offset;   // first element of the piece inside the tensor
+  int length;   // elements, <= kRunPiece
+};
+struct RunTable {
+  RunPiece *pieces = nullptr;  // device
+  int n_pieces = 0;
+  int count = 0;               // parameters covered (must equal the launch's count)
+};
+std::mutex run_mu;
+std::unordered_map<const void *, RunTable> run_tables;  // keyed by the device `number` table
+
+template <int NPTR, class F>
+__global__ __launch_bounds__(kThreads) void multi_tensor_kernel(F f, float *const *p0, float *const *p1,
+                                                               float *const *p2, float *const *p3,
+                                                               const RunPiece *__restrict__ pieces) {
+  const RunPiece piece = pieces[blockIdx.x];
+  float *t0 = p0[piece.tensor] + piece.offset;
+  float *t1 = p1[piece.tensor] + piece.offset;
+  float *t2 = NPTR > 2 ? p2[piece.tensor] + piece.offset : nullptr;
+  float *t3 = NPTR > 2 ? p3[piece.tensor] + piece.offset : nullptr;
+  bool vec = ((reinterpret_cast<uintptr_t>(t0) | reinterpret_cast<uintptr_t>(t1)) & 15u) == 0;
+  if (NPTR > 2) vec = vec && ((reinterpret_cast<uintptr_t>(t2) | reinterpret_cast<uintptr_t>(t3)) & 15u) == 0;
+  const int n4 = vec ? piece.length / 4 : 0;
+  for (int i = threadIdx.x; i < n4; i += kThreads) f.template apply<f32x4>(t0, t1, t2, t3, i);
+  for (int i = n4 * 4 + threadIdx.x; i < piece.length; i += kThreads) f.template apply<float>(t0, t1, t2, t3, i);
+}
+
+struct MultiSgd {
+  float lr;
+  template <class V>
+  __device__ inline void apply(float *w, float *g, float *, float *, int i) const {
+    V *w4 = reinterpret_cast<V *>(w);
+    const V gv = __builtin_nontemporal_load(reinterpret_cast<const V *>(g) + i);
+    w4[i] = w4[i] - lr * gv;
+  }
+};
+struct MultiAdam {
+  float b1, b2, b1t, b2t, e, lr;
+  template <class V>
+  __device__ inline void apply(float *w, float *m, float *v, float *g, int i) const {
+    V *w4 = reinterpret_cast<V *>(w), *m4 = reinterpret_cast<V *>(m), *v4 = reinterpret_cast<V *>(v);
+    const V gi = __builtin_nontemporal_load(reinterpret_cast<const V *>(g) + i);
+    const V mm = m4[i] * b1 + gi * (1.f - b1);
+    const V vv = v4[i] * b2 + gi * gi * (1.f - b2);
+    m4[i] = mm;
+    v4[i] = vv;
+    V root = vv / (1.f - b2t);
+    if constexpr (sizeof(V) == sizeof(float)) {
+      root = sqrtf(root);
+    } else {
+      root.x = sqrtf(root.x); root.y = sqrtf(root.y); root.z = sqrtf(root.z); root.w = sqrtf(root.w);
+    }
+    w4[i] = w4[i] - (lr * mm / (1.f - b1t)) / (root + e);
+  }
+};
+
+// Run table of the launch whose tables start at `number_table`, if its host arrays were runs.
+bool find_run_table(const void *number_table, int count, RunTable &out) {
+  std::lock_guard<std::mutex> g(run_mu);
+  auto it = run_tables.find(number_table);
+  if (it == run_tables.end() || it->second.count != count || it->second.n_pieces == 0) return false;
+  out = it->second;
+  return true;
+}
+
 }  // namespace
 
 extern "C" int DLGpuArraySet(DLArrayHandle arr, float value, void **stream) {
@@ -189,14 +271,14 @@ extern "C" int DLGpuRelu(const DLArrayHandle in, DLArrayHandle out) {
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out), "shape mismatch");
   return launch_ew<OpRelu, true, false>(OpRelu{}, (float *)out->data, (const float *)in->data, nullptr,
-                                        numel(out), nullptr, "DLGpuRelu");
+                                        numel(out), streamless_launch_stream(), "DLGpuRelu");
 }
 
 extern "C" int DLGpuReluGradient(const DLArrayHandle in, const DLArrayHandle grad, DLArrayHandle out) {
   TF_REQUIRE(on_gpu(in) && on_gpu(grad) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out) && same_shape(grad, out), "shape mismatch");
   return launch_ew<OpReluGrad, true, true>(OpReluGrad{}, (float *)out->data, (const float *)in->data,
-                                           (const float *)grad->data, numel(out), nullptr,
+                                           (const float *)grad->data, numel(out), streamless_launch_stream(),
                                            "DLGpuReluGradient");
 }
 
@@ -308,6 +390,28 @@ extern "C" int DLGpuGetIndextoVaribaleNumberCudaPointer(int *index_to_number, in
   *result = (void **)malloc(sizeof(void *) * 2);
   (*result)[0] = d_number;
   (*result)[1] = d_prefix;
+  // the same tables as runs of consecutive offsets inside one tensor, cut into pieces
+  std::vector<RunPiece> pieces;
+  for (int i = 0; i < count;) {
+    int j = i + 1;
+    while (j < count && index_to_number[j] == index_to_number[i] && prefix[j] == prefix[i] + (j - i)) ++j;
+    for (int start = i; start < j; start += kRunPiece)
+      pieces.push_back(RunPiece{index_to_number[i], prefix[i] + (start - i), std::min(kRunPiece, j - start)});
+    i = j;
+  }
+  // worth it only when the pieces are long on average (scattered indices stay with the indexed kernel)
+  if (!pieces.empty() && (int64_t)pieces.size() * 256 <= (int64_t)count + 256 * 1024) {
+    RunTable t;
+    t.n_pieces = (int)pieces.size();
+    t.count = count;
+    if (hipMalloc((void **)&t.pieces, pieces.size() * sizeof(RunPiece)) == hipSuccess &&
+        hipMemcpy(t.pieces, pieces.data(), pieces.size() * sizeof(RunPiece), hipMemcpyHostToDevice) == hipSuccess) {
+      std::lock_guard<std::mutex> g(run_mu);
+      run_tables[d_number] = t;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
   return 0;
 }
 
@@ -344,21 +448,38 @@ extern "C" int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int c
                            const float learning_rate) {
   TF_REQUIRE(n4list && *n4list && indexlist && *indexlist && count >= 0, "bad arguments");
   if (count == 0) return 0;
-  // no stream argument: default stream, ordered against all created streams
-  hipLaunchKernelGGL(adam_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, nullptr,
+  // no stream argument: ordered against all streams that run kernels
+  hipStream_t s = streamless_launch_stream();
+  RunTable runs;
+  if (find_run_table((*indexlist)[0], count, runs)) {
+    hipLaunchKernelGGL((multi_tensor_kernel<4, MultiAdam>), dim3(runs.n_pieces), dim3(kThreads), 0, s,
+                       MultiAdam{b1, b2, b1t, b2t, e, learning_rate}, (float *const *)((*n4list)[0]),
+                       (float *const *)((*n4list)[1]), (float *const *)((*n4list)[2]),
+                       (float *const *)((*n4list)[3]), (const RunPiece *)runs.pieces);
+    return finish(s, "DLGpuAdam_o");
+  }
+  hipLaunchKernelGGL(adam_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, s,
                      (float **)((*n4list)[0]), (float **)((*n4list)[1]), (float **)((*n4list)[2]),
                      (float **)((*n4list)[3]), (const int *)((*indexlist)[0]), (const int *)((*indexlist)[1]), b1,
                      b2, b1t, b2t, e, learning_rate, count);
-  return finish(nullptr, "DLGpuAdam_o");
+  return finish(s, "DLGpuAdam_o");
 }
 
 extern "C" int DLGpuSgd_o(void ****n2list, const void ***indexlist, const int count,
                           const float learning_rate) {
   TF_REQUIRE(n2list && *n2list && indexlist && *indexlist && count >= 0, "bad arguments");
   if (count == 0) return 0;
-  // no stream argument: default stream, ordered against all created streams
-  hipLaunchKernelGGL(sgd_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, nullptr,
+  // no stream argument: ordered against all streams that run kernels
+  hipStream_t s = streamless_launch_stream();
+  RunTable runs;
+  if (find_run_table((*indexlist)[0], count, runs)) {
+    hipLaunchKernelGGL((multi_tensor_kernel<2, MultiSgd>), dim3(runs.n_pieces), dim3(kThreads), 0, s,
+                       MultiSgd{learning_rate}, (float *const *)((*n2list)[0]), (float *const *)((*n2list)[1]),
+                       (float *const *)nullptr, (float *const *)nullptr, (const RunPiece *)runs.pieces);
+    return finish(s, "DLGpuSgd_o");
+  }
+  hipLaunchKernelGGL(sgd_multi_kernel, dim3(grid_for(count)), dim3(kThreads), 0, s,
                      (float **)((*n2list)[0]), (float **)((*n2list)[1]), (const int *)((*indexlist)[0]),
                      (const int *)((*indexlist)[1]), learning_rate, count);
-  return finish(nullptr, "DLGpuSgd_o");
+  return finish(s, "DLGpuSgd_o");
 }

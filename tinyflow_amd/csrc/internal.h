@@ -22,6 +22,7 @@ void pinned_free(void *p);
 
 // ---- streams ----------------------------------------------------------------
 hipStream_t stream_of(void **cell);      // cell written by DLGpuCreatecudaStream; NULL -> default stream
+hipStream_t streamless_launch_stream();  // for entry points without a stream argument
 bool sync_every_op();                    // TINYFLOW_SYNC_EVERY_OP=1
 int finish(hipStream_t s, const char *what);  // launch-error check (+ optional sync)
 

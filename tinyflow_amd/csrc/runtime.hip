@@ -424,6 +424,26 @@ unsigned *fold_tickets(hipStream_t s) {
   return *cell;
 }
 
+// Stream for the entry points that have no stream argument (the reference runs
+// them on the legacy default stream, which is ordered against every other stream).
+// When exactly one stream created here has run kernels, work placed on it is ordered
+// the same way with respect to everything this library enqueues -- behind that
+// stream's earlier kernels, in front of its later ones, and copies on other streams
+// order themselves against it -- without the default stream's wait for all streams,
+// which stalls the host once per call.  Otherwise: the default stream.
+hipStream_t streamless_launch_stream() {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  hipStream_t only = nullptr;
+  int kernel_streams = 0;
+  for (auto &rec : r.streams)
+    if (rec.runs_kernels) {
+      only = rec.stream;
+      ++kernel_streams;
+    }
+  return kernel_streams == 1 ? only : nullptr;
+}
+
 bool sync_every_op() {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);

@@ -8,6 +8,8 @@ as the reference wrappers do.
 """
 import ctypes
 
+import numpy as np
+
 from ._base import _LIB, c_array, check_call
 from . import ndarray as _nd
 
@@ -387,11 +389,23 @@ def adam_compute(output, m, v, b1t, b2t, e, learning_rate, cudaStream):
                               cudaStream))
 
 
+def _int_table(values):
+    """C int array for a list, or the buffer of a numpy array (int32 copy if needed)."""
+    if isinstance(values, np.ndarray):
+        arr = np.ascontiguousarray(values, dtype=np.int32)
+        return arr, arr.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+    arr = c_array(ctypes.c_int, values)
+    return arr, arr
+
+
 def get_index_to_VaribaleNumber_cuda_pointer(index_to_Variable, prefix_list, index_count):
+    """Device tables index -> (tensor number, offset inside the tensor) for the fused
+    optimizers; the two tables may be lists (as the reference passes them) or numpy arrays."""
     result = _cell(3)
-    check_call(_LIB.DLGpuGetIndextoVaribaleNumberCudaPointer(
-        c_array(ctypes.c_int, index_to_Variable), c_array(ctypes.c_int, prefix_list),
-        ctypes.c_int(index_count), result))
+    keep_a, number = _int_table(index_to_Variable)
+    keep_b, offset = _int_table(prefix_list)
+    check_call(_LIB.DLGpuGetIndextoVaribaleNumberCudaPointer(number, offset, ctypes.c_int(index_count), result))
+    del keep_a, keep_b
     return result
 
 
