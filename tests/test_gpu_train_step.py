@@ -215,6 +215,29 @@ def test_fused_bn_relu_executor_is_bit_identical():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("config", ["mlp", "lenet5"])
+def test_known_upstream_scalar_gives_the_bits_of_the_read_back(monkeypatch, config):
+    """The step executor applies the (1,)-shaped upstream gradient of the loss (a
+    ``oneslike`` value) as the constant 1.0 instead of reading it back from the device
+    every step; losses and parameters must have the bits of the read-back path."""
+    from tinyflow_amd import TrainExecute, models
+    runs = []
+    for shortcut in (True, False):
+        if not shortcut:
+            monkeypatch.setattr(TrainExecute, "_known_scalar_compute", lambda node, shapes: None)
+        model, X, y = models.build(config)
+        ex = TrainExecute.TrainExecutor(model.loss, 0.01)
+        ex.init_Variable(dict(model.variables))
+        steps = []
+        for _ in range(3):
+            out = ex.run({model.X: X, model.y_: y})
+            steps.append([o.asnumpy().tobytes() for o in out])
+        runs.append(steps)
+        ex.close()
+    assert runs[0] == runs[1]
+
+
+@pytest.mark.gpu
 def test_fused_update_is_bit_identical_to_per_variable_updates():
     """TrainExecutor(fused_update=True) applies every SGD update of the step with one
     multi-tensor launch behind the last node; losses and parameters over three steps

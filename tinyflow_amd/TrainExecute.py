@@ -115,7 +115,8 @@ class TrainExecutor(object):
             else:
                 node_val = self._alloc(self.node_to_shape_map[node])
                 self.node_to_arr_map[node] = node_val
-            plan.append((node.op.compute, node, input_vals, node_val))
+            plan.append((_known_scalar_compute(node, self.node_to_shape_map) or node.op.compute, node, input_vals,
+                         node_val))
         self._plan = plan
         if fused_sgd:
             self._fused_sgd = _FusedSgd(fused_sgd)
@@ -264,6 +265,37 @@ def find_add_relu_pairs(topo_order, outputs, shapes):
         roles[r] = ("add_relu", s, list(s.inputs))
         roles[a] = ("mask_from_output", s, [r, a.inputs[1], r])
     return roles
+
+
+def _known_scalar_compute(node, shapes):
+    """Plan entry for an Add / Mul node one of whose operands is a (1,)-shaped
+    ``oneslike`` / ``zeroslike`` value, or None.  The op itself reads a (1,) operand
+    back to the host every step and applies it as a constant (reference
+    autodiff.py:302-348, 376-413), which makes the host wait for the whole forward pass
+    at the upstream-gradient scalar of the loss; the value of such a producer is 1.0 or
+    0.0 whatever its input holds, so the constant is known without reading it."""
+    if not isinstance(node.op, (ad.AddOp, ad.MulOp)) or len(node.inputs) != 2:
+        return None
+    a, b = node.inputs
+    if shapes[a] == shapes[b]:
+        return None
+    which = 1 if shapes[b] == (1,) else 0 if shapes[a] == (1,) else None
+    if which is None:
+        return None
+    producer = node.inputs[which]
+    if isinstance(producer.op, ad.OnesLikeOp):
+        constant = 1.0
+    elif isinstance(producer.op, ad.ZerosLikeOp):
+        constant = 0.0
+    else:
+        return None
+    by_const = (gpu_op.matrix_elementwise_add_by_const if isinstance(node.op, ad.AddOp)
+                else gpu_op.matrix_elementwise_multiply_by_const)
+
+    def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+        by_const(input_vals[1 - which], constant, output_val, cudaStream)
+        return 0
+    return compute
 
 
 def _fused_compute(kind, bn):
