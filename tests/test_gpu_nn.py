@@ -37,6 +37,9 @@ POOL_CASES = [
     ((16, 64, 112, 112), "max", 1, 1, 2, 2, 3, 3),  # stem pool at full spatial size
     ((2, 3, 70, 130), "max", 0, 0, 2, 2, 2, 2),     # several tiles per plane, ragged last tile
     ((2, 3, 33, 67), "max", 1, 1, 2, 2, 3, 3),
+    # planes too large to stage whole in LDS: the 16 x 64 tile kernel, ragged last tiles
+    ((2, 2, 150, 130), "max", 0, 0, 2, 2, 2, 2),
+    ((1, 2, 140, 134), "max", 1, 1, 2, 2, 3, 3),
     # windows too large for the one-pass tile kernel: the two-pass kernels
     ((2, 3, 40, 80), "max", 4, 4, 1, 1, 9, 9),      # stride 1: cell kernel
     ((2, 3, 40, 90), "max", 0, 0, 3, 3, 15, 15),    # stride 3: per-element kernel

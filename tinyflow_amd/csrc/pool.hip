@@ -17,6 +17,8 @@
 #include "gemm_core.h"
 #include "internal.h"
 
+#include <type_traits>
+
 #include <algorithm>
 
 using namespace tf;
@@ -201,7 +203,8 @@ __global__ __launch_bounds__(kThreads) void pool_backward_cell_kernel(const unsi
 
 // Max-pool backward in one pass for the window shapes of the reference models
 // (3x3 and 2x2 at stride 2; template arguments, so every loop below unrolls and
-// every division is by a constant).  A workgroup owns a 16 x 64 tile of dx: it
+// every division is by a constant) on planes too large for the whole-plane kernel
+// further down (more than 128 x 128 elements).  A workgroup owns a 16 x 64 tile of dx: it
 // stages the part of x that the tile's windows read in LDS, finds each window's
 // arg-max tap there (same scan as window_argmax, so the same tap), keeps tap and
 // dy per window in LDS, and then every lane gathers four consecutive dx elements
@@ -321,6 +324,113 @@ __global__ __launch_bounds__(kThreads) void pool_max_backward_tile_kernel(const 
 #pragma unroll
     for (int k = 0; k < 4; ++k)
       if (wq + k < pp.W) dst[k] = out[k];
+  }
+}
+
+// One-pass max-pool backward for planes that fit in LDS whole (up to 128 x 128 with at
+// most 4096 windows) and stride-2 windows of 2x2 or 3x3: one workgroup of 1024 lanes per
+// (image, channel) plane
+//   1. stages the plane of x with coalesced loads,
+//   2. finds every window's arg-max tap there (the scan of window_argmax: same tap),
+//   3. clears the plane and lets every window add its dy at its arg-max position, in
+//      four rounds -- windows with (p % 2, q % 2) = (0,0), (0,1), (1,0), (1,1); the
+//      windows of one round are two apart in both directions and cannot touch the
+//      same element, so the adds need no atomics and every element receives its up
+//      to four contributions in a fixed order,
+//   4. streams the plane out as dx.
+// x, dy and dx cross HBM exactly once and the work per element is a fraction of the
+// gather form's (which tests up to four windows per dx element).  Overlapping windows
+// are summed in round order rather than in (p, q) order, so the last bit of such a sum
+// can differ from the other forms; run to run it is the same.
+// VEC: H*W a multiple of 4 and 16-byte aligned planes.
+constexpr int kPlaneMaxFloats = 16384, kPlaneThreads = 1024, kPlaneWindowsPerLane = 4;
+
+template <int FH, int FW, bool VEC>
+__global__ __launch_bounds__(kPlaneThreads) void pool_max_backward_plane_kernel(const float *__restrict__ x,
+                                                                               const float *__restrict__ dy,
+                                                                               float *__restrict__ dx,
+                                                                               PoolParams pp) {
+  constexpr int U = 2, V = 2;
+  extern __shared__ float plane_lds[];
+  typedef float f32x4p __attribute__((ext_vector_type(4)));
+  const int HW = pp.H * pp.W, PQ = pp.P * pp.Q;
+  const int tid = threadIdx.x;
+  const float *plane = x + (int64_t)blockIdx.x * HW;
+  const int n4 = VEC ? HW / 4 : 0;
+  {
+    const f32x4p *src = reinterpret_cast<const f32x4p *>(plane);
+    f32x4p *dst = reinterpret_cast<f32x4p *>(plane_lds);
+    f32x4p v[4];  // 4 x 1024 lanes x 4 floats cover the largest plane
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (tid + k * kPlaneThreads < n4) v[k] = __builtin_nontemporal_load(src + tid + k * kPlaneThreads);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (tid + k * kPlaneThreads < n4) dst[tid + k * kPlaneThreads] = v[k];
+    for (int i = n4 * 4 + tid; i < HW; i += kPlaneThreads) plane_lds[i] = plane[i];
+  }
+  const float *gplane = dy + (int64_t)blockIdx.x * PQ;
+  float gv[kPlaneWindowsPerLane];
+  int target[kPlaneWindowsPerLane];  // element of the plane that receives the window's dy, -1: none
+  int round_of[kPlaneWindowsPerLane];
+#pragma unroll
+  for (int k = 0; k < kPlaneWindowsPerLane; ++k) {
+    const int i = tid + k * kPlaneThreads;
+    gv[k] = i < PQ ? gplane[i] : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kPlaneWindowsPerLane; ++k) {
+    const int i = tid + k * kPlaneThreads;
+    target[k] = -1;
+    round_of[k] = -1;
+    if (i < PQ) {
+      uint32_t p, q;
+      pp.div_q.divmod((uint32_t)i, p, q);
+      round_of[k] = (int)((p & 1u) * 2u + (q & 1u));
+      float best = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < FH; ++r) {
+        const int h = (int)p * U - pp.pad_h + r;
+#pragma unroll
+        for (int sft = 0; sft < FW; ++sft) {
+          const int w = (int)q * V - pp.pad_w + sft;
+          if ((unsigned)h < (unsigned)pp.H && (unsigned)w < (unsigned)pp.W) {
+            const float val = plane_lds[h * pp.W + w];
+            if (val > best || (target[k] < 0 && val == best)) {
+              best = val;
+              target[k] = h * pp.W + w;
+            }
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();  // every window has read its taps: the plane's LDS becomes the dx plane
+  {
+    f32x4p *dst = reinterpret_cast<f32x4p *>(plane_lds);
+    const f32x4p zero = {0.f, 0.f, 0.f, 0.f};
+    for (int i = tid; i < (HW + 3) / 4; i += kPlaneThreads) dst[i] = zero;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int round = 0; round < 4; ++round) {
+    if (FH > U || FW > V || round == 0) {  // disjoint windows need no rounds: all in the first
+#pragma unroll
+      for (int k = 0; k < kPlaneWindowsPerLane; ++k) {
+        const bool mine = (FH > U || FW > V) ? round_of[k] == round : round_of[k] >= 0;
+        if (mine && target[k] >= 0) plane_lds[target[k]] += gv[k];
+      }
+      if (FH > U || FW > V) __syncthreads();
+    }
+  }
+  if (!(FH > U || FW > V)) __syncthreads();
+  float *out_plane = dx + (int64_t)blockIdx.x * HW;
+  {
+    const f32x4p *src = reinterpret_cast<const f32x4p *>(plane_lds);
+    f32x4p *dst = reinterpret_cast<f32x4p *>(out_plane);
+    for (int i = tid; i < n4; i += kPlaneThreads) dst[i] = src[i];
+    for (int i = n4 * 4 + tid; i < HW; i += kPlaneThreads) out_plane[i] = plane_lds[i];
   }
 }
 
@@ -470,6 +580,25 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
     const int tiles_h = cdiv(d->H, kTileH), tiles_w = cdiv(d->W, kTileW);
     const int64_t blocks = (int64_t)d->N * d->C * tiles_h * tiles_w;
     const bool square2 = d->u == 2 && d->v == 2 && d->fh == d->fw && (d->fh == 2 || d->fh == 3);
+    const int HW = d->H * d->W, PQ = d->P * d->Q;
+    if (square2 && HW <= kPlaneMaxFloats && PQ <= kPlaneWindowsPerLane * kPlaneThreads) {
+      // the whole plane fits in LDS: one workgroup per plane, nothing is read twice
+      const bool vec = HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(input->data) |
+                                        reinterpret_cast<uintptr_t>(dinput->data)) & 15u) == 0;
+      const unsigned planes = (unsigned)(d->N * d->C);
+      const size_t lds = (size_t)((HW + 3) / 4 * 4) * sizeof(float);
+      const float *xp = (const float *)input->data, *gp = (const float *)doutput->data;
+      float *dp = (float *)dinput->data;
+      auto run = [&](auto f_c, auto vec_c) {
+        constexpr int F = decltype(f_c)::value;
+        constexpr bool VEC = decltype(vec_c)::value;
+        hipLaunchKernelGGL((pool_max_backward_plane_kernel<F, F, VEC>), dim3(planes), dim3(kPlaneThreads), lds, s, xp, gp,
+                           dp, pp);
+      };
+      if (d->fh == 3) { if (vec) run(std::integral_constant<int, 3>{}, std::true_type{}); else run(std::integral_constant<int, 3>{}, std::false_type{}); }
+      else { if (vec) run(std::integral_constant<int, 2>{}, std::true_type{}); else run(std::integral_constant<int, 2>{}, std::false_type{}); }
+      return finish(s, "DLGpuPooling2DBackward");
+    }
     if (square2 && blocks < ((int64_t)1 << 31)) {
       const bool vec4 = d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(dinput->data) & 15u) == 0;
       const FastDiv div_tiles((uint32_t)(tiles_h * tiles_w)), div_tw((uint32_t)tiles_w);
