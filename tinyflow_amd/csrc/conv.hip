@@ -792,10 +792,18 @@ double predict_us(int M, int N, int K, int bm, int bn, int splits, bool wgrad, b
   const double block_us = a * (g.k_per_split + 9.0);
   const double per_cu = (double)g.blocks() * batch / num_cus();
   const double whole = std::ceil(per_cu);
-  const double rounds = per_cu <= 1.0 ? 1.0 : std::min(whole, per_cu + 0.94);
+  double rounds = per_cu <= 1.0 ? 1.0 : std::min(whole, per_cu + 0.94);
+  // a partial last round whose tiles are cut into pieces and folded in the kernel
+  // (plan_fold) costs about half a round instead of a whole one
+  Geometry folded = g;
+  plan_fold(folded, K, stage_depth(bm, bn), batch);
+  if (g.splits == 1 && folded.fold_pieces > 1) rounds = std::floor(per_cu) + 0.5;
   const double hiding = whole <= 1 ? 0.656 : whole <= 2 ? 0.84 : whole <= 3 ? 0.92 : 1.0;
   double t = rounds * block_us / hiding;
-  if (g.splits > 1) t += (2.0 * g.splits + 1.0) * out_bytes / 6000.0 * 1e-3;
+  // the pieces of a short split are folded by the last workgroup of each tile: no second
+  // launch, and the pieces are read while other tiles still compute
+  if (g.splits > 1)
+    t += (folded.splits == 1 ? 0.6 : 1.0) * (2.0 * g.splits + 1.0) * out_bytes / 6000.0 * 1e-3;
   if (scatter && bm * bn > 4096) t *= 1.0 + 0.164 * (bm * bn / 4096.0 - 1.0);
   return t;
 }

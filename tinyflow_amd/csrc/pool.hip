@@ -434,6 +434,54 @@ __global__ __launch_bounds__(kPlaneThreads) void pool_max_backward_plane_kernel(
   }
 }
 
+// Max-pool forward for the same planes and windows: the plane of x is staged in LDS
+// with coalesced 16-byte loads and every window reads its taps there, so x crosses HBM
+// once (the general kernel fetches each tap from memory, rows of a window a whole image
+// row apart).  The scan order and the comparisons are the general kernel's: same bits.
+template <int FH, int FW, bool VEC>
+__global__ __launch_bounds__(kPlaneThreads) void pool_max_forward_plane_kernel(const float *__restrict__ x,
+                                                                              float *__restrict__ y, PoolParams pp) {
+  constexpr int U = 2, V = 2;
+  extern __shared__ float plane_lds[];
+  typedef float f32x4p __attribute__((ext_vector_type(4)));
+  const int HW = pp.H * pp.W, PQ = pp.P * pp.Q;
+  const int tid = threadIdx.x;
+  const float *plane = x + (int64_t)blockIdx.x * HW;
+  const int n4 = VEC ? HW / 4 : 0;
+  {
+    const f32x4p *src = reinterpret_cast<const f32x4p *>(plane);
+    f32x4p *dst = reinterpret_cast<f32x4p *>(plane_lds);
+    f32x4p v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (tid + k * kPlaneThreads < n4) v[k] = __builtin_nontemporal_load(src + tid + k * kPlaneThreads);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (tid + k * kPlaneThreads < n4) dst[tid + k * kPlaneThreads] = v[k];
+    for (int i = n4 * 4 + tid; i < HW; i += kPlaneThreads) plane_lds[i] = plane[i];
+  }
+  __syncthreads();
+  float *out = y + (int64_t)blockIdx.x * PQ;
+  for (int i = tid; i < PQ; i += kPlaneThreads) {
+    uint32_t p, q;
+    pp.div_q.divmod((uint32_t)i, p, q);
+    float acc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < FH; ++r) {
+      const int h = (int)p * U - pp.pad_h + r;
+#pragma unroll
+      for (int sft = 0; sft < FW; ++sft) {
+        const int w = (int)q * V - pp.pad_w + sft;
+        if ((unsigned)h < (unsigned)pp.H && (unsigned)w < (unsigned)pp.W) {
+          const float val = plane_lds[h * pp.W + w];
+          acc = val > acc ? val : acc;
+        }
+      }
+    }
+    out[i] = acc;
+  }
+}
+
 // Global pooling (the window is the whole, unpadded plane; one output per plane), mean
 // mode: a workgroup stages `planes` consecutive planes -- one contiguous run of memory --
 // in LDS with coalesced loads, then one lane per plane adds its HW values in the order
@@ -541,6 +589,23 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
     const int HW = d->H * d->W, planes = std::min(kThreads, kGlobalFloats / HW);
     hipLaunchKernelGGL(global_mean_forward_kernel, dim3(cdiv(total, planes)), dim3(kThreads), 0, s,
                        (const float *)input->data, (float *)output->data, HW, planes, (int)total);
+    return finish(s, "DLGpuPooling2DForward");
+  }
+  const bool square2 = d->u == 2 && d->v == 2 && d->fh == d->fw && (d->fh == 2 || d->fh == 3);
+  if (d->mode == 0 && square2 && d->H * d->W <= kPlaneMaxFloats) {
+    const int HW = d->H * d->W;
+    const bool vec = HW % 4 == 0 && (reinterpret_cast<uintptr_t>(input->data) & 15u) == 0;
+    const unsigned planes = (unsigned)(d->N * d->C);
+    const size_t lds = (size_t)((HW + 3) / 4 * 4) * sizeof(float);
+    const float *xp = (const float *)input->data;
+    float *yp = (float *)output->data;
+    auto run = [&](auto f_c, auto vec_c) {
+      constexpr int F = decltype(f_c)::value;
+      constexpr bool VEC = decltype(vec_c)::value;
+      hipLaunchKernelGGL((pool_max_forward_plane_kernel<F, F, VEC>), dim3(planes), dim3(kPlaneThreads), lds, s, xp, yp, pp);
+    };
+    if (d->fh == 3) { if (vec) run(std::integral_constant<int, 3>{}, std::true_type{}); else run(std::integral_constant<int, 3>{}, std::false_type{}); }
+    else { if (vec) run(std::integral_constant<int, 2>{}, std::true_type{}); else run(std::integral_constant<int, 2>{}, std::false_type{}); }
     return finish(s, "DLGpuPooling2DForward");
   }
   if (d->mode == 0)
