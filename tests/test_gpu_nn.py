@@ -264,6 +264,27 @@ def test_dropout_backward_needs_its_forward(rt):
 
 
 @pytest.mark.gpu
+def test_dropout_forward_twice_releases_the_first_mask(rt):
+    """A forward whose backward never runs (an evaluation pass) must not leak its mask:
+    the next forward through the same input descriptor releases it, and a backward on
+    the discarded cells is refused."""
+    from tinyflow_amd import gpu_op, ndarray
+    shape = (64, 4096)
+    x = ndarray.array(np.ones(shape, np.float32), rt.ctx)
+    out = ndarray.empty(shape, rt.ctx)
+    inputd = gpu_op.get_input_descriptor(shape, "NCHW")
+    first = gpu_op.dropout_forward(x, out, "NCHW", 0.5, 1, inputd, rt.cudnn, rt.stream)
+    in_use = gpu_op.device_memory_stats()[1]
+    for seed in range(2, 12):
+        last = gpu_op.dropout_forward(x, out, "NCHW", 0.5, seed, inputd, rt.cudnn, rt.stream)
+    assert gpu_op.device_memory_stats()[1] == in_use    # ten more forwards hold one mask, not eleven
+    with pytest.raises(RuntimeError):
+        gpu_op.dropout_backward(x, out, first[0], first[1], rt.cudnn, rt.stream)
+    gpu_op.dropout_backward(x, out, last[0], last[1], rt.cudnn, rt.stream)
+    assert gpu_op.device_memory_stats()[1] < in_use
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("sa,sb", [((3, 2, 4, 5), (3, 7, 4, 5)), ((64, 256, 28, 28), (64, 64, 28, 28)),
                                    ((4, 10), (4, 1)), ((1, 1, 1), (1, 3, 1))])
 def test_concat_forward_and_backward(rt, sa, sb):

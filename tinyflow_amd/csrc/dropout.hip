@@ -27,9 +27,15 @@ constexpr int kThreads = 256;
 constexpr int kMagicInput = 0x7466496e;    // 'tfIn'
 constexpr int kMagicDropout = 0x74664472;  // 'tfDr'
 
+struct DropoutDesc;
 struct InputDesc {
   int magic;
   int64_t count;
+  // mask + list published by the last forward through this descriptor and not yet
+  // consumed by a backward (the binding makes new cells for every forward, so the
+  // descriptor, which lives as long as its node, is where an unconsumed pair is found)
+  DropoutDesc *pending;
+  void **pending_slots;
 };
 
 struct DropoutDesc {
@@ -170,6 +176,17 @@ extern "C" int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle outp
   TF_REQUIRE(numel(input) == in->count && numel(output) == in->count, "arrays do not match the descriptor");
   TF_REQUIRE(dropout >= 0.f && dropout < 1.f, "dropout probability %g outside [0, 1)", (double)dropout);
   hipStream_t s = stream_of(stream);
+  // a forward whose backward never ran (an evaluation-only pass): release its mask and
+  // list before publishing new ones (a backward on the old cells is then refused)
+  // The mask goes back to the pool; the two small host records are only invalidated,
+  // not freed, because the caller's old cells still point at them.
+  if (in->pending) {
+    device_free(in->pending->reserve);
+    in->pending->reserve = nullptr;
+    in->pending->magic = 0;
+    in->pending = nullptr;
+    in->pending_slots = nullptr;
+  }
   const int64_t groups = (in->count + 7) / 8;
   unsigned char *mask = (unsigned char *)device_alloc((size_t)(groups > 0 ? groups : 1));
   if (!mask) {
@@ -186,6 +203,8 @@ extern "C" int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle outp
   slots[0] = d;
   slots[1] = in;
   *cudnnlist = slots;
+  in->pending = d;
+  in->pending_slots = slots;
   if (groups > 0) {
     // drop when the 32-bit draw is below dropout * 2^32
     const double t = (double)dropout * 4294967296.0;
@@ -212,6 +231,10 @@ extern "C" int DLGpuDropoutBackward(const DLArrayHandle doutput, DLArrayHandle d
                        0, s, (const float *)doutput->data, (float *)dinput->data, (unsigned char *)d->reserve,
                        d->count, 0u, 0u, d->scale);
   // the mask and the list are consumed (stream-ordered release), as in the reference
+  if (InputDesc *in = reinterpret_cast<InputDesc *>((*cudnnlist)[1]); in && in->magic == kMagicInput && in->pending == d) {
+    in->pending = nullptr;
+    in->pending_slots = nullptr;
+  }
   device_free(d->reserve);
   *reserveSpace_p = nullptr;
   d->magic = 0;

@@ -175,6 +175,10 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
   const int64_t a_bytes = numel(matA) * 4, b_bytes = numel(matB) * 4;
   TF_REQUIRE(a_bytes < (1ll << 31) && b_bytes < (1ll << 31) && M * N * 4 < (1ll << 31),
              "operands and results of 2 GiB or more are not supported");
+  // the epilogue forms 32-bit byte offsets for every row of a tile, including the rows
+  // of the last tile that lie past M (the buffer bound drops them only if the offset
+  // has not wrapped)
+  TF_REQUIRE((M + 128) * N * 4 < (1ll << 32), "result too wide: (rows + 128) * columns * 4 must stay below 4 GiB");
   hipStream_t s = stream_of(stream);
   if (M == 0 || N == 0) return 0;
   if (K == 0) return DLGpuArraySet(matC, 0.f, stream);
