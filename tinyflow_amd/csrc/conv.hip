@@ -773,38 +773,36 @@ struct ConvPlan {
 // Tile and k-split selection.  Every ResNet/VGG layer offers several workable
 // (tile, splits) pairs and the best one is worth 10-30 % on the small-image stages,
 // so the choice is made by a cost model rather than by a rule of thumb.  The model
-// (microseconds) was fitted to a sweep of all pairs over the ResNet-50 batch-64
-// layers on MI355X (rms error 12 %, its picks within 2 % of the sweep's optimum):
-//   workgroup time   = a(tile) * (k per split + 9), a = 0.0705 / 0.0406 / 0.0229 us
+// (microseconds) was fitted to sweeps of all pairs over the ResNet-50 layers at batch
+// 16 / 64 / 128 and the VGG-16 layers at batch 32 on MI355X, first to the measured
+// times (rms error 14 %), then nudged so that its picks cost least (within 1 % of the
+// sweeps' optimum on ResNet-50 batch 64, 2 % at batch 128):
+//   workgroup time   = a(tile) * (k per split + 24), a = 0.065 / 0.0332 / 0.0178 us
 //                      per reduction step for 128x128 / 64x128 / 64x64
 //   rounds           = workgroups / CUs, rounded up once a CU holds more than one
 //   latency hiding   = a CU that only ever holds 1 / 2 / 3 workgroups runs them at
-//                      0.66 / 0.84 / 0.92 of the rate it reaches with four or more
-//   split-sum pass   = (2 * splits + 1) * output bytes at 6 TB/s
+//                      0.68 / 0.87 / 0.95 of the rate it reaches with four or more
+//   split-sum pass   = (2 * splits + 1) * output bytes at 6.5 TB/s
 // It depends on the problem shape and the CU count only, so a given layer always
-// gets the same plan and results stay bit-reproducible from run to run.
+// gets the same plan and results stay bit-reproducible from run to run.  The batched
+// products of the Winograd forms (batch > 1) keep the constants they were tuned with.
 double predict_us(int M, int N, int K, int bm, int bn, int splits, bool wgrad, bool padded, bool scatter,
                   double out_bytes, int batch = 1) {
   const Geometry g = make_geometry(M, N, K, bm, bn, splits, stage_depth(bm, bn));
-  double a = (bm == 128 && bn == 128) ? 0.0705 : (bm == 64 && bn == 128) ? 0.0406 : 0.0229;
-  if (padded) a *= 1.04;
-  if (wgrad) a *= bm == 128 ? 0.98 : 1.05;
-  const double block_us = a * (g.k_per_split + 9.0);
+  const bool one = batch == 1;
+  double a = (bm == 128 && bn == 128) ? (one ? 0.065 : 0.0705) : (bm == 64 && bn == 128) ? (one ? 0.0332 : 0.0406)
+                                                                                           : (one ? 0.0178 : 0.0229);
+  if (padded) a *= one ? 1.17 : 1.04;
+  if (wgrad) a *= bm == 128 ? (one ? 0.906 : 0.98) : (one ? 1.24 : 1.05);
+  const double block_us = a * (g.k_per_split + (one ? 23.8 : 9.0));
   const double per_cu = (double)g.blocks() * batch / num_cus();
   const double whole = std::ceil(per_cu);
-  double rounds = per_cu <= 1.0 ? 1.0 : std::min(whole, per_cu + 0.94);
-  // a partial last round whose tiles are cut into pieces and folded in the kernel
-  // (plan_fold) costs about half a round instead of a whole one
-  Geometry folded = g;
-  plan_fold(folded, K, stage_depth(bm, bn), batch);
-  if (g.splits == 1 && folded.fold_pieces > 1) rounds = std::floor(per_cu) + 0.5;
-  const double hiding = whole <= 1 ? 0.656 : whole <= 2 ? 0.84 : whole <= 3 ? 0.92 : 1.0;
+  const double rounds = per_cu <= 1.0 ? 1.0 : std::min(whole, per_cu + (one ? 0.85 : 0.94));
+  const double hiding = one ? (whole <= 1 ? 0.675 : whole <= 2 ? 0.865 : whole <= 3 ? 0.953 : 1.0)
+                            : (whole <= 1 ? 0.656 : whole <= 2 ? 0.84 : whole <= 3 ? 0.92 : 1.0);
   double t = rounds * block_us / hiding;
-  // the pieces of a short split are folded by the last workgroup of each tile: no second
-  // launch, and the pieces are read while other tiles still compute
-  if (g.splits > 1)
-    t += (folded.splits == 1 ? 0.6 : 1.0) * (2.0 * g.splits + 1.0) * out_bytes / 6000.0 * 1e-3;
-  if (scatter && bm * bn > 4096) t *= 1.0 + 0.164 * (bm * bn / 4096.0 - 1.0);
+  if (g.splits > 1) t += (2.0 * g.splits + 1.0) * out_bytes / (one ? 6485.0 : 6000.0) * 1e-3;
+  if (scatter && bm * bn > 4096) t *= 1.0 + (one ? 0.045 : 0.164) * (bm * bn / 4096.0 - 1.0);
   return t;
 }
 
