@@ -243,7 +243,7 @@ struct DyAcross {
 struct StoreNCHW {
   float *out;
   int m_extent, n_extent;
-  FastDiv div_hw;
+  FastDiv div_hw;        // pixels per image in the column index (HW, or HW rounded up to 4: ragged segments)
   int HW;
   int64_t split_stride;  // elements between the partial outputs of consecutive k-splits
   struct State {
@@ -258,7 +258,7 @@ struct StoreNCHW {
       const int n = n_wave + 32 * j + (lane & 31);
       uint32_t img, pix;
       div_hw.divmod((uint32_t)(n < n_extent ? n : 0), img, pix);
-      st.col_off[j] = n < n_extent ? (img * (uint32_t)m_extent * (uint32_t)HW + pix) * 4u : OOB;
+      st.col_off[j] = (n < n_extent && pix < (uint32_t)HW) ? (img * (uint32_t)m_extent * (uint32_t)HW + pix) * 4u : OOB;
     }
   }
   __device__ inline void store(const State &st, int m, int /*n*/, int j, float v) const {
@@ -275,6 +275,7 @@ struct StoreScatter {
   FastDiv div_pq, div_q;
   int H, W, u, v;
   bool pairs;  // u = v = 2 with even H and W: every cell is a full, 8-byte aligned 2 x 2 block
+  int pq_valid;  // real P*Q (div_pq may divide by P*Q rounded up to 4: ragged segments)
   struct State {
     int col_base[4];
     int rows[4], cols[4];
@@ -288,7 +289,7 @@ struct StoreScatter {
       div_pq.divmod((uint32_t)(n < n_extent ? n : 0), img, rem);
       div_q.divmod(rem, p, q);
       const int h0 = (int)p * u, w0 = (int)q * v;
-      st.col_base[j] = n < n_extent ? ((int)img * m_extent * H + h0) * W + w0 : -1;
+      st.col_base[j] = (n < n_extent && rem < (uint32_t)pq_valid) ? ((int)img * m_extent * H + h0) * W + w0 : -1;
       st.rows[j] = min(u, H - h0);
       st.cols[j] = min(v, W - w0);
     }
@@ -766,9 +767,20 @@ struct ConvPlan {
   bool a_vec, b_vec;     // operand fetched with the 16-byte loaders (shape permitting)
   int bm, bn, splits;
   int M, N, K;
+  int seg = 0;            // pixels per image as the 16-byte loaders index them: P*Q, or P*Q rounded up
+                          // to a multiple of 4 (ragged segments); 0 when they are not used
   bool winograd = false;  // 3x3 / stride-1 layers: transformed-domain products (bm x bn is their tile)
   int wino_tile = 2;      // F(2x2, 3x3) or F(4x4, 3x3)
 };
+
+// Pixels per image as the 16-byte loaders index a [image][channel][pixel] block: the
+// real count when it is a multiple of 4; otherwise rounded up (ragged segments, see
+// gemm_core.h) as long as the padding columns cost at most an eighth more work.
+int vector_segment(int pixels) {
+  if (pixels % 4 == 0) return pixels;
+  const int padded = (pixels + 3) / 4 * 4;
+  return padded * 8 <= pixels * 9 ? padded : 0;
+}
 
 // Tile and k-split selection.  Every ResNet/VGG layer offers several workable
 // (tile, splits) pairs and the best one is worth 10-30 % on the small-image stages,
@@ -980,7 +992,13 @@ void consider_winograd_wgrad(ConvPlan &p, const ConvDesc *d, double direct_us) {
       if (t[1] == 128 && d->C <= 64) continue;
       for (int splits : cand) {
         if (splits > 1 && (w.Tp / splits < 64 || splits * out_bytes > 256e6)) continue;
-        const double us = predict_us(d->K, d->C, w.Tp, t[0], t[1], splits, false, false, false, out_bytes, w.positions);
+        double us = predict_us(d->K, d->C, w.Tp, t[0], t[1], splits, false, false, false, out_bytes, w.positions);
+        // the kernel that folds the splits and applies G^T . G runs one workgroup per 64
+        // filters; with few filters (64 x 64: 64 workgroups) it cannot pull the partial
+        // sums at the memory rate (about 25 GB/s per workgroup, measured), which is what
+        // the split term of predict_us assumes
+        const double fold_rate = std::min(6.0e6, std::ceil(d->K * (double)d->C / 64.0) * 25.0e3);  // bytes per us
+        if (splits > 1) us += splits * out_bytes * (1.0 / fold_rate - 1.0 / 6.0e6);
         if (us < best) {
           best = us;
           bm = t[0];
@@ -1021,13 +1039,17 @@ ConvPlan plan_forward(const ConvDesc *d) {
   p.N = d->N * d->P * d->Q;
   p.K = d->C * d->R * d->S;
   const bool padded = d->pad_h || d->pad_w;
-  const double direct_us = choose_tile_and_splits(p, false, padded, false, true, 4.0 * p.M * p.N);
-  p.variant = padded ? "fwd_pad" : "fwd_nopad";
-  p.epilogue = "StoreNCHW";
   // filter rows of C*R*S floats; a 1x1 / stride-1 / unpadded input is a plain
   // [image][channel][pixel] block
   p.a_vec = p.K % 4 == 0;
-  p.b_vec = p.a_vec && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1 && (d->P * d->Q) % 4 == 0;
+  p.seg = vector_segment(d->P * d->Q);
+  p.b_vec = p.a_vec && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1 && p.seg != 0 &&
+            (int64_t)d->N * p.seg < (1ll << 31);
+  if (p.b_vec) p.N = d->N * p.seg;  // columns in the loaders' (possibly padded) index space
+  else p.seg = 0;
+  const double direct_us = choose_tile_and_splits(p, false, padded, false, true, 4.0 * p.M * d->N * d->P * d->Q);
+  p.variant = padded ? "fwd_pad" : "fwd_nopad";
+  p.epilogue = "StoreNCHW";
   p.a_loader = p.a_vec ? "Across4" : "PlainAcross";
   p.b_loader = p.b_vec ? "Along4" : "GatherAlong";
   p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
@@ -1049,12 +1071,15 @@ ConvPlan plan_dgrad(const ConvDesc *d) {
   if (RS == 1) {
     p.N = d->N * d->P * d->Q;
     const bool dense = d->u == 1 && d->v == 1;
+    // dy is read compactly, [image][out channel][pixel]
+    p.seg = vector_segment(d->P * d->Q);
+    p.b_vec = p.a_vec && p.seg != 0 && (int64_t)d->N * p.seg < (1ll << 31);
+    p.a_vec = p.b_vec;
+    if (p.b_vec) p.N = d->N * p.seg;
+    else p.seg = 0;
     choose_tile_and_splits(p, false, false, !dense, dense, 4.0 * p.M * d->N * d->H * d->W);
     p.variant = dense ? "dgrad_1x1" : "dgrad_1x1_scatter";
     if (!dense) p.epilogue = "StoreScatter";
-    // dy is read compactly, [image][out channel][pixel]
-    p.b_vec = p.a_vec && (d->P * d->Q) % 4 == 0;
-    p.a_vec = p.b_vec;
   } else {
     p.N = d->N * d->H * d->W;
     if (d->u == 1 && d->v == 1) {
@@ -1081,13 +1106,19 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
   p.N = d->C * d->R * d->S;
   p.K = d->N * d->P * d->Q;
   const bool padded = d->pad_h || d->pad_w;
+  // dy is [image][out channel][pixel]; x is the same kind of block for a 1x1 /
+  // stride-1 / unpadded filter.  Both operands then share the reduction index, which
+  // may be the padded one of ragged segments; a gathered x keeps the real index, so dy
+  // is vectorised next to it only when its segments are whole.
+  const int PQ = d->P * d->Q;
+  p.seg = vector_segment(PQ);
+  p.b_vec = p.seg != 0 && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1 && (int64_t)d->N * p.seg < (1ll << 31);
+  p.a_vec = p.b_vec || PQ % 4 == 0;
+  if (!p.b_vec) p.seg = p.a_vec ? PQ : 0;
+  p.K = d->N * (p.seg ? p.seg : PQ);
   const double direct_us = choose_tile_and_splits(p, true, padded, false, true, 4.0 * p.M * p.N);
   p.variant = padded ? "wgrad_pad" : "wgrad_nopad";
   p.epilogue = "StoreRowMajor";
-  // dy is [image][out channel][pixel]; x is the same kind of block for a 1x1 /
-  // stride-1 / unpadded filter
-  p.a_vec = (d->P * d->Q) % 4 == 0;
-  p.b_vec = p.a_vec && !padded && d->R * d->S == 1 && d->u == 1 && d->v == 1;
   p.a_loader = p.a_vec ? "Across4" : "DyAcross";
   p.b_loader = p.b_vec ? "Across4" : "GatherAcross";
   p.b_mode = p.b_vec ? -1 : padded ? 1 : 0;
@@ -1240,10 +1271,12 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
     return 0;
   }
   char b_args[32];
+  const bool ragged_wgrad = which == 2 && p.b_vec && p.seg != d->P * d->Q;
   if (p.b_mode >= 0) snprintf(b_args, sizeof b_args, "%d, %d, %d", p.bn, bk, p.b_mode);
-  else snprintf(b_args, sizeof b_args, "%d, %d", p.bn, bk);
-  snprintf(name, (size_t)name_len, "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d>, %s<%s>, %s>", p.variant,
-           p.bm, p.bn, p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, p.b_loader, b_args, p.epilogue);
+  else snprintf(b_args, sizeof b_args, ragged_wgrad ? "%d, %d, true" : "%d, %d", p.bn, bk);
+  snprintf(name, (size_t)name_len, "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d%s>, %s<%s>, %s>", p.variant,
+           p.bm, p.bn, p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, ragged_wgrad ? ", true" : "", p.b_loader, b_args,
+           p.epilogue);
   if (flops)
     *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
   return 0;
@@ -1342,17 +1375,21 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
     }
   }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
-  const bool aligned = vec4_ok(filter->data, 0) && vec4_ok(input->data, 0);
+  const int PQ = d->P * d->Q;
+  // (a plan with ragged segments counts its columns in the padded index space, so it
+  // keeps the 16-byte loaders whatever the alignment: they only need 4 bytes)
+  const bool aligned = (vec4_ok(filter->data, 0) && vec4_ok(input->data, 0)) || (plan.seg != 0 && plan.seg != PQ);
   const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
   const uint32_t w_bytes = (uint32_t)(numel(filter) * 4), x_bytes = (uint32_t)(numel(input) * 4);
-  const int PQ = d->P * d->Q;
   with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
-    StoreNCHW ep{partial ? partial : (float *)output->data, M, N, FastDiv((uint32_t)PQ), PQ, numel(output)};
+    // with the 16-byte loader the columns are (image, pixel) in its segment index space
+    const int seg = b_vec ? plan.seg : PQ;
+    StoreNCHW ep{partial ? partial : (float *)output->data, M, N, FastDiv((uint32_t)seg), PQ, numel(output)};
     auto with_b = [&](const auto &al, auto a_is_vec) {
       if constexpr (decltype(a_is_vec)::value) {  // a vectorised input only comes with a vectorised filter
         if (b_vec) {
-          Along4<BN, BK> bl{(const float *)input->data, x_bytes, PQ, N, K, FastDiv((uint32_t)PQ), d->C * PQ};
+          Along4<BN, BK> bl{(const float *)input->data, x_bytes, PQ, N, K, FastDiv((uint32_t)seg), d->C * PQ};
           launch<BM, BN, BK>(al, bl, ep, K, g, s);
           return;
         }
@@ -1445,30 +1482,33 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   float *dst = partial ? partial : (float *)dinput->data;
   const int64_t dx_count = numel(dinput);
 
-  const bool aligned = vec4_ok(wt, 0) && vec4_ok(doutput->data, 0);
+  // (a plan with ragged segments keeps the 16-byte loaders whatever the alignment)
+  const bool aligned = (vec4_ok(wt, 0) && vec4_ok(doutput->data, 0)) || (plan.seg != 0 && plan.seg != PQ);
   const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
   const FastDiv whole(ONE_SEGMENT);
   if (RS == 1) {
     // 1x1 filter (pad 0): compact GEMM over the output pixels + scatter
     const int N = plan.N;
     const int bm = plan.bm, bn = plan.bn;
+    const int seg = (a_vec && b_vec) ? plan.seg : PQ;  // pixels per image in the column index
     with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
       constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
       auto with_epilogue = [&](const auto &al, const auto &bl) {
         if (d->u == 1 && d->v == 1) {
-          StoreNCHW ep{dst, M, N, FastDiv((uint32_t)PQ), PQ, dx_count};
+          StoreNCHW ep{dst, M, N, FastDiv((uint32_t)seg), PQ, dx_count};
           launch<BM, BN, BK>(al, bl, ep, K, g, s);
         } else {
-          StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)PQ), FastDiv((uint32_t)d->Q),
+          StoreScatter ep{(float *)dinput->data, M, N, FastDiv((uint32_t)seg), FastDiv((uint32_t)d->Q),
                           d->H, d->W, d->u, d->v,
                           d->u == 2 && d->v == 2 && d->H % 2 == 0 && d->W % 2 == 0 &&
-                              (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0};
+                              (reinterpret_cast<uintptr_t>(dinput->data) & 7u) == 0,
+                          PQ};
           launch<BM, BN, BK>(al, bl, ep, K, g, s);
         }
       };
       if (a_vec && b_vec) {
         with_epilogue(Along4<BM, BK>{wt, w_bytes, d->C, M, K, whole, 0},
-                      Along4<BN, BK>{(const float *)doutput->data, dy_bytes, PQ, N, K, FastDiv((uint32_t)PQ),
+                      Along4<BN, BK>{(const float *)doutput->data, dy_bytes, PQ, N, K, FastDiv((uint32_t)seg),
                                      d->K * PQ});
       } else {
         with_epilogue(PlainAlong<BM, BK>{wt, w_bytes, d->C, M, K},
@@ -1554,13 +1594,21 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
     dst = partial;
   }
   const bool padded = d->pad_h != 0 || d->pad_w != 0;
-  const bool aligned = vec4_ok(doutput->data, 0) && vec4_ok(input->data, 0);
+  const bool ragged = plan.seg != 0 && plan.seg != PQ;  // both operands in the padded reduction index
+  const bool aligned = (vec4_ok(doutput->data, 0) && vec4_ok(input->data, 0)) || ragged;
   const bool a_vec = plan.a_vec && aligned, b_vec = plan.b_vec && aligned;
   const uint32_t dy_bytes = (uint32_t)(numel(doutput) * 4), x_bytes = (uint32_t)(numel(input) * 4);
   with_tile(bm, bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     if constexpr (BM == BN) {  // only the square tiles are used for grad-filter
       StoreRowMajor ep{dst, N, M, N, (int64_t)M * N};
+      if (ragged) {  // 1x1, stride 1, pixels per image not a multiple of 4: masked 16-byte loads on both sides
+        const FastDiv div_seg((uint32_t)plan.seg);
+        Across4<BM, BK, true> al{(const float *)doutput->data, dy_bytes, PQ, M, K, div_seg, d->K * PQ, PQ};
+        Across4<BN, BK, true> bl{(const float *)input->data, x_bytes, PQ, N, K, div_seg, d->C * PQ, PQ};
+        launch<BM, BN, BK>(al, bl, ep, K, g, s);
+        return;
+      }
       auto with_b = [&](const auto &al, auto a_is_vec) {
         if constexpr (decltype(a_is_vec)::value) {
           if (b_vec) {

@@ -175,6 +175,15 @@ struct PlainAcross {
 // Preconditions, checked by the callers: base 16-byte aligned; ld, inner and outer
 // multiples of 4; the extent along the vectorised direction (d for Along4, k for
 // Across4) a multiple of 4, so that a vector is entirely inside or outside.
+//
+// Ragged segments: a segment whose real length is not a multiple of 4 (the 49 pixels
+// of a 7x7 map) is addressed with `inner` rounded up to the next multiple of 4 while
+// `outer` stays the real distance between segments.  The last vector of a segment
+// then also fetches up to three elements that belong to what follows it in memory
+// (4-byte aligned 16-byte loads are fine for global memory).  For Along4 they land in
+// tile columns that exist only in the padded index space and are dropped by the
+// epilogue; for Across4 they would enter the reduction, so its RAGGED form zeroes
+// every element whose position in the segment is `seg_valid` or more.
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr uint32_t ONE_SEGMENT = 0x80000000u;
 __device__ inline f32x4v buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
@@ -232,7 +241,7 @@ struct Along4 {
   }
 };
 
-template <int D, int BK>
+template <int D, int BK, bool RAGGED = false>
 struct Across4 {
   static constexpr int LPR = BK / 4;            // lanes per d row of the tile
   static constexpr int DSTEP = THREADS / LPR;
@@ -244,6 +253,7 @@ struct Across4 {
   int ld, d_extent, k_extent;
   FastDiv div_inner;
   int outer;
+  int seg_valid = 0;  // RAGGED: real length of a segment
 
   struct State {
     __amdgpu_buffer_rsrc_t rsrc;
@@ -269,7 +279,7 @@ struct Across4 {
     for (int e = 0; e < VPT; ++e) {
       const f32x4v v = buf_load4(st.rsrc, (st.row_off[e] + k_off) | ((st.row_off[e] | k_off) & OOB));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) reg[4 * e + i] = v[i];
+      for (int i = 0; i < 4; ++i) reg[4 * e + i] = (RAGGED && (int)rem + i >= seg_valid) ? 0.f : v[i];
     }
   }
   template <int LD>
