@@ -13,7 +13,9 @@ time; the per-family figures quoted in the design notes come from it):
 ``compare`` asserts err_hip <= k * err_cpu32 (+ one rounding step of the largest
 reference magnitude, so that an exactly representable result cannot make the bound
 zero): the HIP result is no further from the exact answer than a plain fp32 CPU
-evaluation is, up to the stated factor k.
+evaluation is, up to the stated factor k.  It also asserts the literal bar relative to
+that evaluation: the fraction of elements that meet it may trail the fp32 CPU
+evaluation's own fraction by at most 1e-3 (+ one element).
 """
 import json
 import os
@@ -62,6 +64,11 @@ def compare(got, ref64, ref32, family, what, k, assert_ratio=True):
             "%s: largest error %.3g exceeds %g x the fp32 CPU evaluation's %.3g" % (what, hip_max, k, cpu_max)
         assert hip_rms <= k * cpu_rms + floor, \
             "%s: rms error %.3g exceeds %g x the fp32 CPU evaluation's %.3g" % (what, hip_rms, k, cpu_rms)
+        # the literal bar: no element count worth mentioning may fail it that the fp32 CPU evaluation passes
+        margin = 1e-3 + 1.0 / max(1, rec["elements"])
+        assert rec["literal"] >= rec["literal_cpu32"] - margin, \
+            "%s: %.6f of the elements meet rtol 1e-3 / atol 1e-5, the fp32 CPU evaluation reaches %.6f" % (
+                what, rec["literal"], rec["literal_cpu32"])
     return rec
 
 
