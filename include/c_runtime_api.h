@@ -257,6 +257,13 @@ int DLGpuConvolutionDescribeKernel(void ***list, int which, char *name, int name
  * can time exactly the kernel a profiler lists under the described symbol. */
 int DLGpuConvolutionTimeNextKernel(void *start_event, void *stop_event);
 
+/* No counterpart in the reference: introspection for tests.  A Winograd forward call
+ * may keep its transformed input for the grad-filter call of the same step on the same,
+ * unmodified input array (any entry point that writes or frees the array drops it).
+ * Reports how many such blocks were kept and how many were taken over since the
+ * library was loaded, and how many are held right now; any pointer may be NULL. */
+int DLGpuKeptByproductCounts(long long *kept_blocks, long long *taken_blocks, int *held_now);
+
 /* ----------------------------------------------------------------- pooling */
 
 /* out = 1 + (in + 2*pad - window) / stride.

@@ -195,6 +195,76 @@ def test_conv_gradients_are_deterministic(rt):
     np.testing.assert_array_equal(outs[0][1], outs[1][1])
 
 
+def _kept_counts():
+    import ctypes
+    from tinyflow_amd import _base
+    kept, taken, held = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
+    assert _base._LIB.DLGpuKeptByproductCounts(ctypes.byref(kept), ctypes.byref(taken), ctypes.byref(held)) == 0
+    return kept.value, taken.value, held.value
+
+
+def test_kept_transformed_input_follows_the_input_array(rt, monkeypatch):
+    """A Winograd forward call keeps its transformed input for the grad-filter call on the
+    same array.  Grad-filter must give the bits it gives without the kept block, and must
+    not use a block whose source array was overwritten, freed or replaced in between."""
+    from tinyflow_amd import gpu_op, ndarray
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "4")
+    rng = np.random.RandomState(23)
+    xs, ws = (4, 64, 28, 28), (64, 64, 3, 3)
+    x1 = rng.normal(0, 1, xs).astype(np.float32)
+    x2 = rng.normal(0, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.05, ws).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(xs, ws, "NCHW", "SAME", 1, 1)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gw, gdy = _gpu(w, rt), _gpu(dy, rt)
+    gy = ndarray.empty(out_shape, rt.ctx)
+
+    def grad_filter(gx):
+        gdw = ndarray.empty(ws, rt.ctx)
+        assert gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream) == 0
+        return gdw.asnumpy()
+
+    gx = _gpu(x1, rt)
+    want1 = grad_filter(gx)                    # nothing kept yet: transforms x itself
+    gx2 = _gpu(x2, rt)
+    want2 = grad_filter(gx2)
+    assert not np.array_equal(want1, want2)
+
+    # forward then grad-filter on the untouched array: the kept block is taken over
+    kept0, taken0, _ = _kept_counts()
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    kept1, taken1, held1 = _kept_counts()
+    assert kept1 == kept0 + 1 and held1 >= 1
+    np.testing.assert_array_equal(grad_filter(gx), want1)
+    assert _kept_counts()[1] == taken1 + 1
+
+    # the array is overwritten between the two calls: the block is dropped, x2 is transformed
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    gx[:] = x2
+    taken = _kept_counts()[1]
+    np.testing.assert_array_equal(grad_filter(gx), want2)
+    assert _kept_counts()[1] == taken
+
+    # an in-place kernel writes the array
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    gpu_op.matrix_elementwise_multiply_by_const(gx, 2.0, gx, rt.stream)
+    np.testing.assert_array_equal(grad_filter(gx), grad_filter(_gpu(2.0 * x2, rt)))
+
+    # the array is freed and another one (most likely at the same address) takes its place
+    gx = _gpu(x1, rt)
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    del gx
+    gx = _gpu(x2, rt)
+    taken = _kept_counts()[1]
+    np.testing.assert_array_equal(grad_filter(gx), want2)
+    assert _kept_counts()[1] == taken
+
+    # grad-filter on another array than the one forward saw
+    gx = _gpu(x1, rt)
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    np.testing.assert_array_equal(grad_filter(gx2), want2)
+
+
 # ResNet-50 batch-64 layer shapes, one per kernel family: (C, H, K, R, padding, stride)
 FULL_SIZE_LAYERS = [
     (128, 28, 128, 3, "SAME", 1),    # 3x3, Winograd 4x4 tiles

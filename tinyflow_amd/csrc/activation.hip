@@ -44,6 +44,7 @@ extern "C" int DLGpuActivationGetCudnnlist(const int *input_shapes, const int si
 
 extern "C" int DLGpuActivationForward(const DLArrayHandle input, DLArrayHandle output, int activationMode,
                                       void ***list, void **handle, void **stream) {
+  announce_write(output);
   (void)handle;
   ActDesc *d = desc_from_list<ActDesc>(list, kMagicAct);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuActivationGetCudnnlist");
@@ -68,6 +69,7 @@ extern "C" int DLGpuActivationForward(const DLArrayHandle input, DLArrayHandle o
 extern "C" int DLGpuActivationBackward(const DLArrayHandle input, DLArrayHandle dinput,
                                        const DLArrayHandle output, const DLArrayHandle doutput,
                                        int activationMode, void ***list, void **handle, void **stream) {
+  announce_write(dinput);
   (void)handle;
   ActDesc *d = desc_from_list<ActDesc>(list, kMagicAct);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuActivationGetCudnnlist");

@@ -463,6 +463,7 @@ extern "C" int DLGpuBatchNormalizationForward(const DLArrayHandle input, DLArray
                                               int batchNormMode, int n, void **mean_p, void **Variance_p,
                                               void ***list, void **handle, int *memorytoSaving,
                                               void **stream) {
+  announce_write(output);
   return bn_forward_impl(input, output, batchNormMode, n, mean_p, Variance_p, list, handle, memorytoSaving, stream,
                          false, "DLGpuBatchNormalizationForward");
 }
@@ -474,6 +475,7 @@ extern "C" int DLGpuBatchNormalizationReluForward(const DLArrayHandle input, DLA
                                                   int batchNormMode, int n, void **mean_p, void **Variance_p,
                                                   void ***list, void **handle, int *memorytoSaving,
                                                   void **stream) {
+  announce_write(output);
   return bn_forward_impl(input, output, batchNormMode, n, mean_p, Variance_p, list, handle, memorytoSaving, stream,
                          true, "DLGpuBatchNormalizationReluForward");
 }
@@ -558,6 +560,7 @@ extern "C" int DLGpuBatchNormalizationBackward(const DLArrayHandle input, const 
                                                DLArrayHandle dinput, int batchNormMode, void **mean_p,
                                                void **Variance_p, void ***list, void **handle,
                                                int *memorytoSaving, void **stream) {
+  announce_write(dinput);
   return bn_backward_impl(input, doutput, dinput, batchNormMode, mean_p, Variance_p, list, handle, memorytoSaving,
                           stream, false, "DLGpuBatchNormalizationBackward");
 }
@@ -570,6 +573,7 @@ extern "C" int DLGpuBatchNormalizationReluBackward(const DLArrayHandle input, co
                                                    DLArrayHandle dinput, int batchNormMode, void **mean_p,
                                                    void **Variance_p, void ***list, void **handle,
                                                    int *memorytoSaving, void **stream) {
+  announce_write(dinput);
   return bn_backward_impl(input, doutput, dinput, batchNormMode, mean_p, Variance_p, list, handle, memorytoSaving,
                           stream, true, "DLGpuBatchNormalizationReluBackward");
 }

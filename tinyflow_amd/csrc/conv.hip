@@ -1129,17 +1129,35 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
 // Runs the planned Winograd form: filter and input transforms, the batched products,
 // the output transform.  Scratch follows the usual convention (shortfall reported
 // through memorytoSaving, nothing written).
-int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in, const float *filter,
+// The grad-filter call of a training step needs the transformed input V = B^T x B of the
+// forward call of that step again.  Once a descriptor has seen a grad-filter call in a
+// Winograd form, its forward calls with the same tile put V in a block of its own and
+// keep it (keep_set: valid until anything writes to x), and grad-filter takes it over
+// instead of transforming x a second time.  The values are the ones it would compute.
+// Nothing is kept under a device-memory budget or with TINYFLOW_KEEP_TRANSFORMED_INPUT=0.
+bool keeping_transformed_input() {
+  static const bool on = [] {
+    const char *e = getenv("TINYFLOW_KEEP_TRANSFORMED_INPUT");
+    return !(e && *e && atoi(e) == 0);
+  }();
+  return on && !device_budget_active();
+}
+
+int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in, const float *filter,
                  float *out, int *memorytoSaving, hipStream_t s) {
   WinoShape w;
   if (!wino_shape(d, dgrad, w, false, plan.wino_tile)) return -1;
   const size_t bytes = (w.u_elems + w.v_elems + w.m_elems) * sizeof(float);
-  float *U = (float *)device_alloc(bytes);
+  float *kept_V = nullptr;
+  if (!dgrad && d->grad_filter_tile == w.tile && keeping_transformed_input())
+    kept_V = (float *)device_alloc(w.v_elems * sizeof(float));  // no room: this call keeps nothing
+  float *U = (float *)device_alloc(bytes - (kept_V ? w.v_elems * sizeof(float) : 0));
   if (!U) {
+    if (kept_V) device_free(kept_V);
     if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
-  float *V = U + w.u_elems, *Mt = V + w.v_elems;
+  float *V = kept_V ? kept_V : U + w.u_elems, *Mt = kept_V ? U + w.u_elems : V + w.v_elems;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
   const dim3 fgrid(cdiv(d->K * d->C, 256)), igrid(cdiv(w.Tp, 256), w.Cr), ogrid(cdiv(w.T, 256), w.Mo), block(256);
   auto transforms_in = [&](auto tile_c) {
@@ -1184,24 +1202,35 @@ int run_winograd(const ConvDesc *d, bool dgrad, const ConvPlan &plan, const floa
     hipLaunchKernelGGL(wino_output_kernel<4>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
                        div_tiles, div_tw, w.T, w.Tp, rows_vec);
   device_free(U);
+  if (kept_V) {
+    d->kept_stream = s;
+    d->kept_tile = w.tile;
+    keep_set(&d->kept_v, kept_V, in, (size_t)d->N * d->C * d->H * d->W * sizeof(float));
+  }
   return 0;
 }
 
-int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, const float *dy, float *dw,
+int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const float *dy, float *dw,
                        int *memorytoSaving, hipStream_t s) {
   WinoShape w;
   if (!wino_shape(d, false, w, true, plan.wino_tile)) return -1;
+  d->grad_filter_tile = w.tile;
+  // V of this step's forward call, if it is still there, belongs to this x, this tile and this stream
+  float *kept_V = nullptr;
+  if (d->kept_tile == w.tile && d->kept_stream == s && keeping_transformed_input())
+    kept_V = (float *)keep_take(&d->kept_v, x);
   const int KC = d->K * d->C;
   const int bk = stage_depth(plan.bm, plan.bn);
   const Geometry g = make_geometry(d->K, d->C, w.Tp, plan.bm, plan.bn, plan.splits, bk);
   const size_t du_elems = (size_t)g.splits * w.positions * KC;
-  const size_t bytes = (w.v_elems + w.m_elems + du_elems) * sizeof(float);
-  float *V = (float *)device_alloc(bytes);
-  if (!V) {
+  const size_t bytes = ((kept_V ? 0 : w.v_elems) + w.m_elems + du_elems) * sizeof(float);
+  float *scratch = (float *)device_alloc(bytes);
+  if (!scratch) {
+    if (kept_V) device_free(kept_V);
     if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
-  float *dM = V + w.v_elems, *dU = dM + w.m_elems;
+  float *V = kept_V ? kept_V : scratch, *dM = kept_V ? scratch : scratch + w.v_elems, *dU = dM + w.m_elems;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
   const bool rows_vec = d->Q % w.tile == 0 && (reinterpret_cast<uintptr_t>(dy) & (uintptr_t)(4 * w.tile - 1)) == 0;
   const dim3 block(256);
@@ -1212,7 +1241,9 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
       row16 = d->pad_w == 1 && d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
       halves = !row16 && d->pad_w == 1 && d->W % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0;
     }
-    if (row16)
+    if (kept_V)
+      ;  // V is the forward call's
+    else if (row16)
       hipLaunchKernelGGL((wino_input_kernel<4, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
                          div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
     else if (halves)
@@ -1238,7 +1269,8 @@ int run_winograd_wgrad(const ConvDesc *d, const ConvPlan &plan, const float *x, 
     hipLaunchKernelGGL(wino_dfilter_kernel<2>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
   else
     hipLaunchKernelGGL(wino_dfilter_kernel<4>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
-  device_free(V);
+  device_free(scratch);
+  if (kept_V) device_free(kept_V);
   return 0;
 }
 
@@ -1342,6 +1374,7 @@ static int check_conv_arrays(const ConvDesc *d, const DLArray *x, const DLArray 
 extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArrayHandle filter,
                                          DLArrayHandle output, void ***list, void **handle,
                                          int *memorytoSaving, void **stream) {
+  announce_write(output);
   (void)handle;
   ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
@@ -1422,6 +1455,7 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
 extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLArrayHandle doutput,
                                             const DLArrayHandle filter, DLArrayHandle dinput, void ***list,
                                             void **handle, int *memorytoSaving, void **stream) {
+  announce_write(dinput);
   (void)handle;
   ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");
@@ -1555,6 +1589,7 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
 extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const DLArrayHandle doutput,
                                               const DLArrayHandle filter, DLArrayHandle dfilter, void ***list,
                                               void **handle, int *memorytoSaving, void **stream) {
+  announce_write(dfilter);
   (void)handle;
   ConvDesc *d = desc_from_list<ConvDesc>(list, kMagicConv);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuConvolution2DForwardGetOutShape");

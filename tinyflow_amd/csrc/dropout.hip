@@ -167,6 +167,7 @@ extern "C" int DLGpuGetInputDescriptor(const int *input_shapes, int sizeofshape,
 extern "C" int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle output, int dataformat, float dropout,
                                    int seed, void **reserveSpace_p, void ***inputd, void ***cudnnlist,
                                    void **handle, int *memorytoSaving, void **stream) {
+  announce_write(output);
   (void)dataformat;
   (void)handle;
   InputDesc *in = desc_from_list<InputDesc>(inputd, kMagicInput);
@@ -218,6 +219,7 @@ extern "C" int DLGpuDropoutForward(const DLArrayHandle input, DLArrayHandle outp
 
 extern "C" int DLGpuDropoutBackward(const DLArrayHandle doutput, DLArrayHandle dinput, void **reserveSpace_p,
                                     void ***cudnnlist, void **handle, void **stream) {
+  announce_write(dinput);
   (void)handle;
   DropoutDesc *d = desc_from_list<DropoutDesc>(cudnnlist, kMagicDropout);
   TF_REQUIRE(d, "list was not created by DLGpuDropoutForward (or was consumed already)");
@@ -246,6 +248,7 @@ extern "C" int DLGpuDropoutBackward(const DLArrayHandle doutput, DLArrayHandle d
 
 extern "C" int DLGpuConcatForward(const DLArrayHandle input1, const DLArrayHandle input2, DLArrayHandle output,
                                   void **stream) {
+  announce_write(output);
   int64_t outer, ca, cb;
   if (concat_geometry(input1, input2, outer, ca, cb) != 0) return -1;
   TF_REQUIRE(on_gpu(output) && numel(output) == numel(input1) + numel(input2), "output has the wrong size");
@@ -277,10 +280,12 @@ static int concat_backward(const DLArray *input1, const DLArray *input2, const D
 
 extern "C" int DLGpuConcataBackward(const DLArrayHandle input1, const DLArrayHandle input2,
                                     const DLArrayHandle doutput, DLArrayHandle dinput1, void **stream) {
+  announce_write(dinput1);
   return concat_backward(input1, input2, doutput, dinput1, false, stream, "DLGpuConcataBackward");
 }
 
 extern "C" int DLGpuConcatbBackward(const DLArrayHandle input1, const DLArrayHandle input2,
                                     const DLArrayHandle doutput, DLArrayHandle dinput2, void **stream) {
+  announce_write(dinput2);
   return concat_backward(input1, input2, doutput, dinput2, true, stream, "DLGpuConcatbBackward");
 }

@@ -213,6 +213,7 @@ bool find_run_table(const void *number_table, int count, RunTable &out) {
 }  // namespace
 
 extern "C" int DLGpuArraySet(DLArrayHandle arr, float value, void **stream) {
+  announce_write(arr);
   TF_REQUIRE(on_gpu(arr), "array must live on the GPU");
   hipStream_t s = stream_of(stream);
   return launch_ew<OpSet, false, false>(OpSet{value}, (float *)arr->data, nullptr, nullptr, numel(arr), s,
@@ -221,6 +222,7 @@ extern "C" int DLGpuArraySet(DLArrayHandle arr, float value, void **stream) {
 
 extern "C" int DLGpuMatrixElementwiseAdd(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
                                          void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
   return launch_ew<OpAdd, true, true>(OpAdd{}, (float *)out->data, (const float *)a->data,
@@ -232,6 +234,7 @@ extern "C" int DLGpuMatrixElementwiseAdd(const DLArrayHandle a, const DLArrayHan
 // the ReLU that follows it, in one pass (12 bytes per element instead of 20).
 extern "C" int DLGpuMatrixElementwiseAddRelu(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
                                              void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
   return launch_ew<OpAddRelu, true, true>(OpAddRelu{}, (float *)out->data, (const float *)a->data,
@@ -241,6 +244,7 @@ extern "C" int DLGpuMatrixElementwiseAddRelu(const DLArrayHandle a, const DLArra
 
 extern "C" int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle in, float val, DLArrayHandle out,
                                                 void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out), "shape mismatch");
   return launch_ew<OpAddC, true, false>(OpAddC{val}, (float *)out->data, (const float *)in->data, nullptr,
@@ -249,6 +253,7 @@ extern "C" int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle in, float va
 
 extern "C" int DLGpuMatrixElementwiseMultiply(const DLArrayHandle a, const DLArrayHandle b, DLArrayHandle out,
                                               void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(a) && on_gpu(b) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(a, out) && same_shape(b, out), "shape mismatch");
   return launch_ew<OpMul, true, true>(OpMul{}, (float *)out->data, (const float *)a->data,
@@ -258,6 +263,7 @@ extern "C" int DLGpuMatrixElementwiseMultiply(const DLArrayHandle a, const DLArr
 
 extern "C" int DLGpuMatrixMultiplyByConst(const DLArrayHandle in, float val, DLArrayHandle out,
                                           void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out), "shape mismatch");
   return launch_ew<OpMulC, true, false>(OpMulC{val}, (float *)out->data, (const float *)in->data, nullptr,
@@ -268,6 +274,7 @@ extern "C" int DLGpuMatrixMultiplyByConst(const DLArrayHandle in, float val, DLA
 // ordered after all work already enqueued on the blocking streams created by
 // DLGpuCreatecudaStream and before any work enqueued on them later.
 extern "C" int DLGpuRelu(const DLArrayHandle in, DLArrayHandle out) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out), "shape mismatch");
   return launch_ew<OpRelu, true, false>(OpRelu{}, (float *)out->data, (const float *)in->data, nullptr,
@@ -275,6 +282,7 @@ extern "C" int DLGpuRelu(const DLArrayHandle in, DLArrayHandle out) {
 }
 
 extern "C" int DLGpuReluGradient(const DLArrayHandle in, const DLArrayHandle grad, DLArrayHandle out) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(grad) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(same_shape(in, out) && same_shape(grad, out), "shape mismatch");
   return launch_ew<OpReluGrad, true, true>(OpReluGrad{}, (float *)out->data, (const float *)in->data,
@@ -283,6 +291,7 @@ extern "C" int DLGpuReluGradient(const DLArrayHandle in, const DLArrayHandle gra
 }
 
 extern "C" int DLGpuSgdUpdate(DLArrayHandle w, const DLArrayHandle g, float lr, void **stream) {
+  announce_write(w);
   TF_REQUIRE(on_gpu(w) && on_gpu(g), "arrays must live on the GPU");
   TF_REQUIRE(numel(w) == numel(g), "parameter and gradient differ in size");
   return launch_ew<OpSgd, true, true>(OpSgd{lr}, (float *)w->data, (const float *)w->data,
@@ -291,6 +300,7 @@ extern "C" int DLGpuSgdUpdate(DLArrayHandle w, const DLArrayHandle g, float lr, 
 
 extern "C" int DLGpuCross(const DLArrayHandle x, const DLArrayHandle y, DLArrayHandle out, float b,
                           void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(x) && on_gpu(y) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(numel(x) == numel(out) && numel(y) == numel(out), "shape mismatch");
   return launch_ew<OpCross, true, true>(OpCross{b}, (float *)out->data, (const float *)x->data,
@@ -299,6 +309,7 @@ extern "C" int DLGpuCross(const DLArrayHandle x, const DLArrayHandle y, DLArrayH
 
 extern "C" int DLGpuCrossBackward(const DLArrayHandle x, const DLArrayHandle y, const DLArrayHandle dout,
                                   DLArrayHandle out, float b, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(x) && on_gpu(y) && on_gpu(dout) && on_gpu(out), "arrays must live on the GPU");
   const int64_t n = numel(out);
   TF_REQUIRE(numel(x) == n && numel(y) == n && numel(dout) == n, "shape mismatch");
@@ -310,6 +321,7 @@ extern "C" int DLGpuCrossBackward(const DLArrayHandle x, const DLArrayHandle y, 
 }
 
 extern "C" int DLGpuBroadcastTo0(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   const int64_t in_count = numel(in), n = numel(out);
   TF_REQUIRE(in_count > 0 && in_count <= INT32_MAX, "bad input size");
@@ -328,6 +340,7 @@ extern "C" int DLGpuBroadcastTo0(const DLArrayHandle in, DLArrayHandle out, void
 }
 
 extern "C" int DLGpuBroadcastTo1(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(in->ndim == 1 && out->ndim >= 2 && in->shape[0] == out->shape[1],
              "input must be (C,) and output (N, C, ...)");
@@ -354,6 +367,8 @@ extern "C" int DLGpuBroadcastTo1(const DLArrayHandle in, DLArrayHandle out, void
 
 extern "C" int DLGpuAdam_mv(DLArrayHandle m, DLArrayHandle v, const DLArrayHandle g, float b1, float b2,
                             void **stream) {
+  announce_write(m);
+  announce_write(v);
   TF_REQUIRE(on_gpu(m) && on_gpu(v) && on_gpu(g), "arrays must live on the GPU");
   const int64_t n = numel(g);
   TF_REQUIRE(numel(m) == n && numel(v) == n, "shape mismatch");
@@ -366,6 +381,7 @@ extern "C" int DLGpuAdam_mv(DLArrayHandle m, DLArrayHandle v, const DLArrayHandl
 
 extern "C" int DLGpuAdam(DLArrayHandle w, const DLArrayHandle m, const DLArrayHandle v, float b1t, float b2t,
                          float e, float lr, void **stream) {
+  announce_write(w);
   TF_REQUIRE(on_gpu(w) && on_gpu(m) && on_gpu(v), "arrays must live on the GPU");
   const int64_t n = numel(w);
   TF_REQUIRE(numel(m) == n && numel(v) == n, "shape mismatch");
@@ -446,6 +462,7 @@ extern "C" int DLGpuGetN4CudaPointer(void **output, void **m, void **v, void **g
 extern "C" int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int count, const float b1,
                            const float b2, const float b1t, const float b2t, const float e,
                            const float learning_rate) {
+  note_write_everything();  // the pointer tables name the written tensors, not their sizes
   TF_REQUIRE(n4list && *n4list && indexlist && *indexlist && count >= 0, "bad arguments");
   if (count == 0) return 0;
   // no stream argument: ordered against all streams that run kernels
@@ -467,6 +484,7 @@ extern "C" int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int c
 
 extern "C" int DLGpuSgd_o(void ****n2list, const void ***indexlist, const int count,
                           const float learning_rate) {
+  note_write_everything();  // the pointer tables name the written tensors, not their sizes
   TF_REQUIRE(n2list && *n2list && indexlist && *indexlist && count >= 0, "bad arguments");
   if (count == 0) return 0;
   // no stream argument: ordered against all streams that run kernels

@@ -58,6 +58,22 @@ inline int shortfall(size_t bytes) {
 // Number of compute units of the current device (256 on MI355X).
 int num_cus();
 
+// ---- by-products kept from one call to a later one (runtime.hip) ----------------
+// An op may keep a device block that it derived from an input array (the transformed
+// input of a Winograd forward call) for a later call on the same input.  Such a block
+// is valid only while the input's bytes are unchanged, so every entry point announces
+// the arrays it is about to write (or free) before it does anything else, and the
+// registry drops what was derived from them.  All device memory behind this ABI is
+// written through these entry points, which is what makes the rule complete.
+void keep_set(void **slot, void *block, const void *src, size_t src_bytes);  // replaces what the slot held
+void *keep_take(void **slot, const void *src);  // the block if it is still valid for `src` (caller frees), else null
+void note_write(const void *ptr, size_t bytes);
+void note_write_everything();
+bool device_budget_active();  // a device-memory limit is set: keep nothing
+inline void announce_write(const DLArray *a) {
+  if (a && a->data && a->ctx.device_type == kGPU) note_write(a->data, (size_t)numel(a) * sizeof(float));
+}
+
 }  // namespace tf
 
 #define TF_REQUIRE(cond, ...)                                  \
@@ -101,6 +117,12 @@ struct ConvDesc {
   int K, R, S;         // filter (K output channels, C input channels)
   int P, Q;            // output spatial
   int pad_h, pad_w, u, v;
+  // Winograd forms: the transformed input V of the last forward call, kept for the
+  // grad-filter call of the same step, which needs exactly this array (see keep_set).
+  void *kept_v = nullptr;
+  hipStream_t kept_stream = nullptr;
+  int kept_tile = 0;
+  int grad_filter_tile = 0;  // tile of the last grad-filter call that ran in a Winograd form (0: none yet)
 };
 
 struct PoolDesc {

@@ -164,6 +164,7 @@ int choose_splits(int tiles, int K, int min_k) {
 
 extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
                                    bool transposeB, DLArrayHandle matC, void **handle, void **stream) {
+  announce_write(matC);
   (void)handle;
   TF_REQUIRE(on_gpu(matA) && on_gpu(matB) && on_gpu(matC), "arrays must live on the GPU");
   TF_REQUIRE(matA->ndim == 2 && matB->ndim == 2 && matC->ndim == 2, "operands must be 2-D");

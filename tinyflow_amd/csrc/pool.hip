@@ -574,6 +574,7 @@ extern "C" int DLGpuPooling2DForwardGetOutShape(const int *input_shapes, int *ou
 
 extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle output, void ***list,
                                      void **handle, void **stream) {
+  announce_write(output);
   (void)handle;
   PoolDesc *d = desc_from_list<PoolDesc>(list, kMagicPool);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuPooling2DForwardGetOutShape");
@@ -620,6 +621,7 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
 extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHandle output,
                                       const DLArrayHandle doutput, DLArrayHandle dinput, void ***list,
                                       void **handle, void **stream) {
+  announce_write(dinput);
   (void)handle;
   PoolDesc *d = desc_from_list<PoolDesc>(list, kMagicPool);
   TF_REQUIRE(d, "descriptor list was not created by DLGpuPooling2DForwardGetOutShape");

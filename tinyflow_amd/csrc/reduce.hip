@@ -299,6 +299,7 @@ int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hip
 }  // namespace
 
 extern "C" int DLGpuReduceSumAxisZero(const DLArrayHandle in, DLArrayHandle out) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(in->ndim >= 1, "input needs at least one dim");
   const int64_t A = in->shape[0];
@@ -344,6 +345,7 @@ float *fixed_scratch_of_current_device(const char *what) {
 }  // namespace
 
 extern "C" int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(in->ndim >= 1, "input needs at least one dim");
   const int64_t A = in->shape[0];
@@ -360,6 +362,7 @@ extern "C" int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle in, DLArrayHand
 }
 
 extern "C" int DLGpuBroadcastToBackward0(const DLArrayHandle in, DLArrayHandle out) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   const int64_t B = numel(out);
   TF_REQUIRE(B > 0 && numel(in) % B == 0, "output size must divide input size");
@@ -374,6 +377,7 @@ extern "C" int DLGpuBroadcastToBackward0(const DLArrayHandle in, DLArrayHandle o
 }
 
 extern "C" int DLGpuBroadcastToBackward1(const DLArrayHandle in, DLArrayHandle out) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(out->ndim == 1 && in->ndim >= 2 && out->shape[0] == in->shape[1],
              "input must be (N, C, ...) and output (C,)");
@@ -408,6 +412,7 @@ extern "C" int DLGReduceSumGetCudnnlist(const int *input_shapes, const int *outp
 
 extern "C" int DLGpuReduceSum(const DLArrayHandle in, DLArrayHandle out, void ***list, void **handle,
                               int *memorytoSaving, void **stream) {
+  announce_write(out);
   (void)handle;
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   ReduceDesc *d = desc_from_list<ReduceDesc>(list, kMagicReduce);
@@ -447,6 +452,7 @@ extern "C" int DLGpuReduceSum(const DLArrayHandle in, DLArrayHandle out, void **
 }
 
 extern "C" int DLGpuSoftmax(const DLArrayHandle in, DLArrayHandle out, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(in) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(in->ndim == 2 && same_shape(in, out), "softmax needs matching 2-D arrays");
   const int64_t rows = in->shape[0];
@@ -460,6 +466,7 @@ extern "C" int DLGpuSoftmax(const DLArrayHandle in, DLArrayHandle out, void **st
 
 extern "C" int DLGpuSoftmaxCrossEntropy(const DLArrayHandle logits, const DLArrayHandle labels,
                                         DLArrayHandle out, void **stream) {
+  announce_write(out);
   TF_REQUIRE(on_gpu(logits) && on_gpu(labels) && on_gpu(out), "arrays must live on the GPU");
   TF_REQUIRE(logits->ndim == 2 && same_shape(logits, labels), "logits and labels must be matching 2-D arrays");
   TF_REQUIRE(numel(out) == 1, "output must hold one element");

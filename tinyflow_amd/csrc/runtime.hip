@@ -10,6 +10,7 @@
 //   * ops do not block the host; copies order themselves after enqueued work.
 #include "internal.h"
 
+#include <atomic>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -525,7 +526,89 @@ extern "C" int DLArrayAlloc(const index_t *shape, index_t ndim_in, DLContext ctx
   return 0;
 }
 
+// ---- by-products kept across calls ---------------------------------------------------
+namespace {
+struct Kept {
+  const char *lo, *hi;  // bytes of the source array
+  void **slot;          // the owner's pointer to the kept block; cleared when the block is dropped
+};
+std::mutex kept_mu;
+std::vector<Kept> kept;
+std::atomic<int> kept_count{0};
+std::atomic<long long> kept_total{0}, taken_total{0};  // blocks registered / handed to a later call
+
+// with kept_mu held
+void drop_at(size_t i) {
+  if (*kept[i].slot) device_free(*kept[i].slot);
+  *kept[i].slot = nullptr;
+  kept[i] = kept.back();
+  kept.pop_back();
+  kept_count.store((int)kept.size(), std::memory_order_release);
+}
+}  // namespace
+
+namespace tf {
+
+void keep_set(void **slot, void *block, const void *src, size_t src_bytes) {
+  std::lock_guard<std::mutex> g(kept_mu);
+  for (size_t i = 0; i < kept.size(); ++i)
+    if (kept[i].slot == slot) {
+      drop_at(i);
+      break;
+    }
+  *slot = block;
+  kept_total.fetch_add(1, std::memory_order_relaxed);
+  kept.push_back({(const char *)src, (const char *)src + src_bytes, slot});
+  kept_count.store((int)kept.size(), std::memory_order_release);
+}
+
+void *keep_take(void **slot, const void *src) {
+  if (kept_count.load(std::memory_order_acquire) == 0) return nullptr;
+  std::lock_guard<std::mutex> g(kept_mu);
+  for (size_t i = 0; i < kept.size(); ++i)
+    if (kept[i].slot == slot) {
+      if (kept[i].lo != (const char *)src) return nullptr;
+      void *block = *slot;
+      *slot = nullptr;
+      drop_at(i);
+      taken_total.fetch_add(1, std::memory_order_relaxed);
+      return block;
+    }
+  return nullptr;
+}
+
+void note_write(const void *ptr, size_t bytes) {
+  if (kept_count.load(std::memory_order_acquire) == 0) return;
+  const char *lo = (const char *)ptr, *hi = lo + bytes;
+  std::lock_guard<std::mutex> g(kept_mu);
+  for (size_t i = 0; i < kept.size();)
+    if (lo < kept[i].hi && kept[i].lo < hi) drop_at(i);
+    else ++i;
+}
+
+void note_write_everything() {
+  if (kept_count.load(std::memory_order_acquire) == 0) return;
+  std::lock_guard<std::mutex> g(kept_mu);
+  while (!kept.empty()) drop_at(kept.size() - 1);
+}
+
+bool device_budget_active() {
+  Runtime &r = rt();
+  std::lock_guard<std::mutex> g(r.mu);
+  return r.dev_limit != 0;
+}
+
+}  // namespace tf
+
+extern "C" int DLGpuKeptByproductCounts(long long *kept_blocks, long long *taken_blocks, int *held_now) {
+  if (kept_blocks) *kept_blocks = kept_total.load(std::memory_order_relaxed);
+  if (taken_blocks) *taken_blocks = taken_total.load(std::memory_order_relaxed);
+  if (held_now) *held_now = kept_count.load(std::memory_order_acquire);
+  return 0;
+}
+
 extern "C" int DLArrayFree(DLArrayHandle handle) {
+  announce_write(handle);
   if (!handle) return 0;
   if (handle->data) {
     if (handle->ctx.device_type == kGPU) device_free(handle->data);
@@ -584,6 +667,7 @@ extern "C" int DLArrayCopyWaitsForCompletion(int kind, int stream_runs_kernels_f
 }
 
 extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
+  announce_write(to);
   TF_REQUIRE(from && to && from->data && to->data, "null array");
   const size_t bytes = array_bytes(from);
   TF_REQUIRE(bytes == array_bytes(to), "size mismatch (%zu vs %zu bytes)", bytes, array_bytes(to));
@@ -620,6 +704,7 @@ extern "C" int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamH
 // will later fill the array with DLArrayCopyIntoFresh: the copy then waits for the
 // work that was enqueued up to this call at most, not up to the copy.
 extern "C" int DLArrayPrepareFresh(DLArrayHandle arr) {
+  announce_write(arr);
   TF_REQUIRE(arr && arr->data && arr->ctx.device_type == kGPU, "not a device array");
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
@@ -639,6 +724,7 @@ extern "C" int DLArrayPrepareFresh(DLArrayHandle arr) {
 // copy waits for everything enqueued, like DLArrayCopyFromTo) -- so the copy overlaps
 // with whatever the compute stream is doing.  Returns after the copy has completed.
 extern "C" int DLArrayCopyIntoFresh(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
+  announce_write(to);
   TF_REQUIRE(from && to && from->data && to->data && stream, "null argument");
   TF_REQUIRE(from->ctx.device_type == kCPU && to->ctx.device_type == kGPU, "host to device only");
   const size_t bytes = array_bytes(from);
@@ -657,6 +743,7 @@ extern "C" int getInt(int *intp) { return intp ? *intp : 0; }
 // is bounded by the physical card): bytes <= 0 removes the limit.  Cached blocks
 // are given back until the budget holds; arrays in use are not touched.
 extern "C" int DLGpuSetDeviceMemoryLimit(int64_t bytes) {
+  note_write_everything();  // nothing is kept from call to call under a budget
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
   r.init();
@@ -711,6 +798,7 @@ extern "C" int DLGpuCreatecudaStream(void **cell) {
 
 extern "C" int DLGpuDestroycudaStream(void **cell) {
   TF_REQUIRE(cell, "null cell");
+  note_write_everything();  // kept blocks are ordered by the stream that made them
   hipStream_t s = reinterpret_cast<hipStream_t>(*cell);
   hipEvent_t ev = nullptr;
   bool found = false;
