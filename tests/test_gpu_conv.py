@@ -265,6 +265,58 @@ def test_kept_transformed_input_follows_the_input_array(rt, monkeypatch):
     np.testing.assert_array_equal(grad_filter(gx2), want2)
 
 
+def test_kept_transformed_filter_follows_the_filter_array(rt, monkeypatch):
+    """A Winograd forward call also writes the transformed filter that grad-data needs and
+    keeps it.  Grad-data must give the bits it gives without the kept block, and must not
+    use a block whose filter was updated in between."""
+    from tinyflow_amd import gpu_op, ndarray
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "4")
+    rng = np.random.RandomState(29)
+    xs, ws = (4, 64, 28, 28), (128, 64, 3, 3)
+    x = rng.normal(0, 1, xs).astype(np.float32)
+    w1 = rng.normal(0, 0.05, ws).astype(np.float32)
+    g = rng.normal(0, 0.05, ws).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(xs, ws, "NCHW", "SAME", 1, 1)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gdy, gg = _gpu(x, rt), _gpu(dy, rt), _gpu(g, rt)
+    gy = ndarray.empty(out_shape, rt.ctx)
+
+    def grad_data(gw):
+        gdx = ndarray.empty(xs, rt.ctx)
+        assert gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream) == 0
+        return gdx.asnumpy()
+
+    gw = _gpu(w1, rt)
+    want1 = grad_data(gw)                      # nothing kept yet
+    gw2 = _gpu(w1 - 0.5 * g, rt)
+    want2 = grad_data(gw2)
+    assert not np.array_equal(want1, want2)
+
+    kept0, taken0, _ = _kept_counts()
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    assert _kept_counts()[0] >= kept0 + 1
+    taken = _kept_counts()[1]
+    np.testing.assert_array_equal(grad_data(gw), want1)
+    assert _kept_counts()[1] == taken + 1
+
+    # the update of the filter comes between forward and grad-data: the block is dropped
+    assert gpu_op.convolution_2d_forward(gx, gw, gy, lst, rt.cudnn, rt.stream) == 0
+    gpu_op.sgd_update(gw, gg, 0.5, rt.stream)
+    taken = _kept_counts()[1]
+    np.testing.assert_array_equal(grad_data(gw), want2)
+    assert _kept_counts()[1] == taken
+
+    # forward itself gives the same bits with and without the second output
+    y_with = gy.asnumpy()
+    gw3 = _gpu(w1, rt)
+    assert gpu_op.convolution_2d_forward(gx, gw3, gy, lst, rt.cudnn, rt.stream) == 0
+    y1 = gy.asnumpy()
+    _, lst_fresh = gpu_op.convolution_2d_forward_get_out_shape(xs, ws, "NCHW", "SAME", 1, 1)
+    assert gpu_op.convolution_2d_forward(gx, gw3, gy, lst_fresh, rt.cudnn, rt.stream) == 0
+    np.testing.assert_array_equal(gy.asnumpy(), y1)
+    assert y_with.shape == y1.shape
+
+
 # ResNet-50 batch-64 layer shapes, one per kernel family: (C, H, K, R, padding, stride)
 FULL_SIZE_LAYERS = [
     (128, 28, 128, 3, "SAME", 1),    # 3x3, Winograd 4x4 tiles

@@ -370,6 +370,7 @@ struct Wino<2> {
   }
   // G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]
   __device__ static inline void g(const float (&f)[3], float (&u)[4]) {
+#pragma clang fp contract(off)  // the same bits wherever this is inlined (a kept block must equal a fresh one)
     u[0] = f[0];
     u[1] = 0.5f * (f[0] + f[1] + f[2]);
     u[2] = 0.5f * (f[0] - f[1] + f[2]);
@@ -416,6 +417,7 @@ struct Wino<4> {
   // G = [64/81 0 0; -128/243 -32/81 -8/27; -128/243 32/81 -8/27; 32/243 16/81 8/27;
   //      32/243 -16/81 8/27; 0 0 1]
   __device__ static inline void g(const float (&f)[3], float (&u)[6]) {
+#pragma clang fp contract(off)  // the same bits wherever this is inlined (a kept block must equal a fresh one)
     const float e1 = (-128.f / 243.f) * f[0] - (8.f / 27.f) * f[2], o1 = (32.f / 81.f) * f[1];
     const float e2 = (32.f / 243.f) * f[0] + (8.f / 27.f) * f[2], o2 = (16.f / 81.f) * f[1];
     u[0] = (64.f / 81.f) * f[0];
@@ -455,30 +457,40 @@ struct Wino<4> {
 // U[pos][k][c] = (G g G^T)[pos], one lane per filter g = w[k][c] (grad-data: rotated by
 // 180 degrees).  Forward reads U as [mo = k][cr = c], grad-data as its transpose
 // [cr = k][mo = c].
+// With `U_rot` the same launch also writes the transform of the rotated filter there
+// (what a later grad-data call of the same step needs), from the nine taps it has loaded.
 template <int TILE>
 __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ w, float *__restrict__ U,
-                                                         int K, int C, bool for_dgrad) {
+                                                         int K, int C, bool for_dgrad,
+                                                         float *__restrict__ U_rot = nullptr) {
   constexpr int A = Wino<TILE>::A;
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= K * C) return;
-  float t[A][3];  // G g, column by column
+  float taps[9];
 #pragma unroll
-  for (int q = 0; q < 3; ++q) {
-    float col[3], u[A];
-#pragma unroll
-    for (int r = 0; r < 3; ++r) col[r] = w[(int64_t)idx * 9 + (for_dgrad ? (2 - r) * 3 + (2 - q) : r * 3 + q)];
-    Wino<TILE>::g(col, u);
-#pragma unroll
-    for (int i = 0; i < A; ++i) t[i][q] = u[i];
-  }
+  for (int q = 0; q < 9; ++q) taps[q] = w[(int64_t)idx * 9 + q];
   const int64_t plane = (int64_t)K * C;
+  auto transform = [&](bool rotated, float *dst) {
+    float t[A][3];  // G g, column by column
 #pragma unroll
-  for (int i = 0; i < A; ++i) {
-    float u[A];
-    Wino<TILE>::g(t[i], u);
+    for (int q = 0; q < 3; ++q) {
+      float col[3], u[A];
 #pragma unroll
-    for (int j = 0; j < A; ++j) U[(i * A + j) * plane + idx] = u[j];
-  }
+      for (int r = 0; r < 3; ++r) col[r] = rotated ? taps[(2 - r) * 3 + (2 - q)] : taps[r * 3 + q];
+      Wino<TILE>::g(col, u);
+#pragma unroll
+      for (int i = 0; i < A; ++i) t[i][q] = u[i];
+    }
+#pragma unroll
+    for (int i = 0; i < A; ++i) {
+      float u[A];
+      Wino<TILE>::g(t[i], u);
+#pragma unroll
+      for (int j = 0; j < A; ++j) dst[(i * A + j) * plane + idx] = u[j];
+    }
+  };
+  transform(for_dgrad, U);
+  if (U_rot) transform(true, U_rot);
 }
 
 // V[pos][cr][t] = (B^T d B)[pos]; d is the patch of in[image][cr] whose corner is
@@ -1151,18 +1163,35 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
   float *kept_V = nullptr;
   if (!dgrad && d->grad_filter_tile == w.tile && keeping_transformed_input())
     kept_V = (float *)device_alloc(w.v_elems * sizeof(float));  // no room: this call keeps nothing
-  float *U = (float *)device_alloc(bytes - (kept_V ? w.v_elems * sizeof(float) : 0));
-  if (!U) {
+  // The transformed filter: a forward call also writes the one grad-data will want (a block
+  // of its own, valid until anything writes to the filter); grad-data takes that over.
+  float *U_for_dgrad = nullptr, *U_kept = nullptr;
+  if (dgrad) d->grad_data_tile = w.tile;
+  if (dgrad && d->kept_u_tile == w.tile && d->kept_u_stream == s && keeping_transformed_input())
+    U_kept = (float *)keep_take(&d->kept_u, filter);
+  if (!dgrad && d->grad_data_tile == w.tile && keeping_transformed_input())
+    U_for_dgrad = (float *)device_alloc(w.u_elems * sizeof(float));
+  const size_t own = bytes - (kept_V ? w.v_elems * sizeof(float) : 0) - (U_kept ? w.u_elems * sizeof(float) : 0);
+  float *scratch = (float *)device_alloc(own);
+  if (!scratch) {
     if (kept_V) device_free(kept_V);
+    if (U_for_dgrad) device_free(U_for_dgrad);
+    if (U_kept) device_free(U_kept);
     if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
-  float *V = kept_V ? kept_V : U + w.u_elems, *Mt = kept_V ? U + w.u_elems : V + w.v_elems;
+  float *next = scratch;
+  float *U = U_kept ? U_kept : next;
+  if (!U_kept) next += w.u_elems;
+  float *V = kept_V ? kept_V : next;
+  if (!kept_V) next += w.v_elems;
+  float *Mt = next;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
   const dim3 fgrid(cdiv(d->K * d->C, 256)), igrid(cdiv(w.Tp, 256), w.Cr), ogrid(cdiv(w.T, 256), w.Mo), block(256);
   auto transforms_in = [&](auto tile_c) {
     constexpr int TILE = decltype(tile_c)::value;
-    hipLaunchKernelGGL(wino_filter_kernel<TILE>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad);
+    if (!U_kept)
+      hipLaunchKernelGGL(wino_filter_kernel<TILE>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad, U_for_dgrad);
     if constexpr (TILE == 4) {
       if (w.pad_w == 1 && w.in_w % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0) {
         hipLaunchKernelGGL((wino_input_kernel<4, true>), igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles,
@@ -1201,11 +1230,17 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
   else
     hipLaunchKernelGGL(wino_output_kernel<4>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
                        div_tiles, div_tw, w.T, w.Tp, rows_vec);
-  device_free(U);
+  device_free(scratch);
+  if (U_kept) device_free(U_kept);
   if (kept_V) {
     d->kept_stream = s;
     d->kept_tile = w.tile;
     keep_set(&d->kept_v, kept_V, in, (size_t)d->N * d->C * d->H * d->W * sizeof(float));
+  }
+  if (U_for_dgrad) {
+    d->kept_u_stream = s;
+    d->kept_u_tile = w.tile;
+    keep_set(&d->kept_u, U_for_dgrad, filter, (size_t)d->K * d->C * 9 * sizeof(float));
   }
   return 0;
 }

@@ -123,6 +123,12 @@ struct ConvDesc {
   hipStream_t kept_stream = nullptr;
   int kept_tile = 0;
   int grad_filter_tile = 0;  // tile of the last grad-filter call that ran in a Winograd form (0: none yet)
+  // the same for the transformed filter of grad-data (the filter rotated by 180 degrees),
+  // which the forward call's filter transform writes along with its own
+  void *kept_u = nullptr;
+  hipStream_t kept_u_stream = nullptr;
+  int kept_u_tile = 0;
+  int grad_data_tile = 0;    // tile of the last grad-data call that ran in a Winograd form (0: none yet)
 };
 
 struct PoolDesc {
