@@ -317,6 +317,73 @@ def test_kept_transformed_filter_follows_the_filter_array(rt, monkeypatch):
     assert y_with.shape == y1.shape
 
 
+@pytest.mark.parametrize("shape", [(4, 64, 28, 28, 64), (3, 32, 14, 14, 48), (2, 16, 7, 9, 24)],
+                         ids=lambda s: "x".join(str(v) for v in s))
+def test_shared_dy_transform_of_the_two_gradients(rt, monkeypatch, shape):
+    """Grad-data and grad-filter of a padded 3x3 layer both transform dy; whichever runs
+    first writes the other's form too.  Either order gives the bits of the separate
+    passes, and a dy overwritten between the two calls is transformed again."""
+    from tinyflow_amd import gpu_op, ndarray
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", "4")
+    N, C, H, W, K = shape
+    rng = np.random.RandomState(31)
+    xs, ws = (N, C, H, W), (K, C, 3, 3)
+    x = rng.normal(0, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.05, ws).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(xs, ws, "NCHW", "SAME", 1, 1)
+    dy1 = rng.normal(0, 1, out_shape).astype(np.float32)
+    dy2 = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gw = _gpu(x, rt), _gpu(w, rt)
+
+    def grad_data(gdy):
+        gdx = ndarray.empty(xs, rt.ctx)
+        assert gpu_op.convolution_backward_data(gx, gdy, gw, gdx, lst, rt.cudnn, rt.stream) == 0
+        return gdx.asnumpy()
+
+    def grad_filter(gdy):
+        gdw = ndarray.empty(ws, rt.ctx)
+        assert gpu_op.convolution_backward_filter(gx, gdy, gw, gdw, lst, rt.cudnn, rt.stream) == 0
+        return gdw.asnumpy()
+
+    def fresh(fn, dy):
+        """The call on a descriptor that has seen nothing yet: no sharing."""
+        nonlocal lst
+        keep = lst
+        _, lst = gpu_op.convolution_2d_forward_get_out_shape(xs, ws, "NCHW", "SAME", 1, 1)
+        out = fn(_gpu(dy, rt))
+        lst = keep
+        return out
+
+    want_dx1, want_dw1 = fresh(grad_data, dy1), fresh(grad_filter, dy1)
+    want_dx2, want_dw2 = fresh(grad_data, dy2), fresh(grad_filter, dy2)
+    gdy = _gpu(dy1, rt)
+    grad_filter(gdy), grad_data(gdy)        # the descriptor now knows both forms
+
+    # grad-filter first: it leaves grad-data's transform
+    taken = _kept_counts()[1]
+    np.testing.assert_array_equal(grad_filter(gdy), want_dw1)
+    np.testing.assert_array_equal(grad_data(gdy), want_dx1)
+    assert _kept_counts()[1] == taken + 1
+    # grad-data first
+    np.testing.assert_array_equal(grad_data(gdy), want_dx1)
+    np.testing.assert_array_equal(grad_filter(gdy), want_dw1)
+    assert _kept_counts()[1] == taken + 2
+    # dy changes between the two calls
+    np.testing.assert_array_equal(grad_filter(gdy), want_dw1)
+    gdy[:] = dy2
+    np.testing.assert_array_equal(grad_data(gdy), want_dx2)
+    gdy[:] = dy1
+    np.testing.assert_array_equal(grad_filter(gdy), want_dw1)
+    assert _kept_counts()[1] == taken + 2
+    # the other call comes with another dy (grad-data first takes what the last grad-filter left for dy1)
+    gdy2 = _gpu(dy2, rt)
+    np.testing.assert_array_equal(grad_data(gdy), want_dx1)
+    assert _kept_counts()[1] == taken + 3
+    np.testing.assert_array_equal(grad_data(gdy), want_dx1)      # leaves grad-filter's form of dy1
+    np.testing.assert_array_equal(grad_filter(gdy2), want_dw2)
+    assert _kept_counts()[1] == taken + 3
+
+
 # ResNet-50 batch-64 layer shapes, one per kernel family: (C, H, K, R, padding, stride)
 FULL_SIZE_LAYERS = [
     (128, 28, 128, 3, "SAME", 1),    # 3x3, Winograd 4x4 tiles

@@ -363,6 +363,7 @@ struct Wino<2> {
   static constexpr int A = 4;
   // B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
   __device__ static inline void bt(const float (&d)[4], float (&t)[4]) {
+#pragma clang fp contract(off)
     t[0] = d[0] - d[2];
     t[1] = d[1] + d[2];
     t[2] = d[2] - d[1];
@@ -383,6 +384,7 @@ struct Wino<2> {
   }
   // the transposes, for grad-filter: A y and G^T u
   __device__ static inline void a(const float (&y)[2], float (&m)[4]) {
+#pragma clang fp contract(off)
     m[0] = y[0];
     m[1] = y[0] + y[1];
     m[2] = y[0] - y[1];
@@ -405,6 +407,7 @@ struct Wino<4> {
   // B^T = [81/64 0 -45/16 0 1 0; 0 -27/16 -9/4 3/4 1 0; 0 27/16 -9/4 -3/4 1 0;
   //        0 -27/32 -9/16 3/2 1 0; 0 27/32 -9/16 -3/2 1 0; 0 81/64 0 -45/16 0 1]
   __device__ static inline void bt(const float (&d)[6], float (&t)[6]) {
+#pragma clang fp contract(off)  // the same bits in every kernel this is inlined into
     const float e1 = d[4] - 2.25f * d[2], o1 = 0.75f * d[3] - 1.6875f * d[1];
     const float e2 = d[4] - 0.5625f * d[2], o2 = 1.5f * d[3] - 0.84375f * d[1];
     t[0] = 1.265625f * d[0] - 2.8125f * d[2] + d[4];
@@ -437,6 +440,7 @@ struct Wino<4> {
   }
   // the transposes, for grad-filter: A y and G^T u
   __device__ static inline void a(const float (&y)[4], float (&m)[6]) {
+#pragma clang fp contract(off)  // the same bits in every kernel this is inlined into
     const float e1 = y[0] + 0.5625f * y[2], o1 = 0.75f * y[1] + 0.421875f * y[3];
     const float e2 = y[0] + 2.25f * y[2], o2 = 1.5f * y[1] + 3.375f * y[3];
     m[0] = y[0];
@@ -499,10 +503,14 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
 // ROW16 (TILE 4 only; pad_w = 1): the four middle columns of a patch row start at a
 // multiple of 4 and are fetched as one 16-byte load (W a multiple of 4, `in` 16-byte
 // aligned) or, with `halves`, as two 8-byte loads (W even, `in` 8-byte aligned).
-template <int TILE, bool ROW16 = false, bool HALVES = false>
+// WITH_DM (padding 1 on both sides, so that the patch's inner TILE x TILE block is the
+// output tile of the same index): the input is a dy, and the launch also writes what
+// grad-filter wants of it, dM[pos][cr][t] = (A y A^T)[pos] with y that inner block --
+// grad-data and grad-filter of one layer then read dy once between them.
+template <int TILE, bool ROW16 = false, bool HALVES = false, bool WITH_DM = false>
 __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
                                                         int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
-                                                        int pad_w, int T, int Tp) {
+                                                        int pad_w, int T, int Tp, float *__restrict__ dM = nullptr) {
   static_assert(!ROW16 || TILE == 4, "ROW16 is the 6-wide patch whose columns 1..4 start at a multiple of 4");
   constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
@@ -573,6 +581,26 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
     Wino<TILE>::bt(r[i], o);
 #pragma unroll
     for (int j = 0; j < A; ++j) dst[(i * A + j) * plane_sz] = o[j];
+  }
+  if constexpr (WITH_DM) {
+    float q[A][TILE];  // A y, column by column
+#pragma unroll
+    for (int b = 0; b < TILE; ++b) {
+      float col[TILE], o[A];
+#pragma unroll
+      for (int a = 0; a < TILE; ++a) col[a] = d[a + 1][b + 1];
+      Wino<TILE>::a(col, o);
+#pragma unroll
+      for (int i = 0; i < A; ++i) q[i][b] = o[i];
+    }
+    float *dst2 = dM + (int64_t)cr * Tp + t;
+#pragma unroll
+    for (int i = 0; i < A; ++i) {
+      float o[A];
+      Wino<TILE>::a(q[i], o);
+#pragma unroll
+      for (int j = 0; j < A; ++j) dst2[(i * A + j) * plane_sz] = o[j];
+    }
   }
 }
 
@@ -1147,6 +1175,38 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
 // keep it (keep_set: valid until anything writes to x), and grad-filter takes it over
 // instead of transforming x a second time.  The values are the ones it would compute.
 // Nothing is kept under a device-memory budget or with TINYFLOW_KEEP_TRANSFORMED_INPUT=0.
+// Launches the input transform x -> V (and, with dM, the grad-filter form of the same
+// array, see WITH_DM) in the variant the row length and alignment allow.
+void launch_wino_input(int tile, const float *in, float *V, float *dM, int Cr, int H, int W, int pad_h, int pad_w,
+                       const FastDiv &div_tiles, const FastDiv &div_tw, int T, int Tp, hipStream_t s) {
+  const dim3 grid(cdiv(Tp, 256), Cr), block(256);
+  if (tile == 2) {
+    hipLaunchKernelGGL(wino_input_kernel<2>, grid, block, 0, s, in, V, Cr, H, W, div_tiles, div_tw, pad_h, pad_w, T, Tp,
+                       nullptr);
+    return;
+  }
+  const bool row16 = pad_w == 1 && W % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  const bool halves = !row16 && pad_w == 1 && W % 2 == 0 && (reinterpret_cast<uintptr_t>(in) & 7u) == 0;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, in, V, Cr, H, W, div_tiles, div_tw, pad_h, pad_w, T, Tp, dM);
+  };
+  if (dM) {
+    if (row16) go(wino_input_kernel<4, true, false, true>);
+    else if (halves) go(wino_input_kernel<4, true, true, true>);
+    else go(wino_input_kernel<4, false, false, true>);
+  } else {
+    if (row16) go(wino_input_kernel<4, true, false, false>);
+    else if (halves) go(wino_input_kernel<4, true, true, false>);
+    else go(wino_input_kernel<4, false, false, false>);
+  }
+}
+
+// dy of a 3x3 / stride-1 layer padded by 1: grad-data's patches and grad-filter's tiles
+// have the same index, so one pass over dy can serve both (F(4x4) forms of both)
+bool dy_transforms_shareable(const ConvDesc *d) {
+  return d->pad_h == 1 && d->pad_w == 1 && d->H == d->P && d->W == d->Q;
+}
+
 bool keeping_transformed_input() {
   static const bool on = [] {
     const char *e = getenv("TINYFLOW_KEEP_TRANSFORMED_INPUT");
@@ -1171,43 +1231,41 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
     U_kept = (float *)keep_take(&d->kept_u, filter);
   if (!dgrad && d->grad_data_tile == w.tile && keeping_transformed_input())
     U_for_dgrad = (float *)device_alloc(w.u_elems * sizeof(float));
-  const size_t own = bytes - (kept_V ? w.v_elems * sizeof(float) : 0) - (U_kept ? w.u_elems * sizeof(float) : 0);
+  // dy: grad-filter may have left grad-data's transform of it, or will want its own
+  float *V_kept = nullptr, *dM_for_wgrad = nullptr;
+  if (dgrad && w.tile == 4 && dy_transforms_shareable(d) && keeping_transformed_input()) {
+    if (d->kept_dy_for == 1 && d->kept_dy_tile == 4 && d->kept_dy_stream == s)
+      V_kept = (float *)keep_take(&d->kept_dy, in);
+    if (!V_kept && d->grad_filter_tile == 4) dM_for_wgrad = (float *)device_alloc(w.v_elems * sizeof(float));
+  }
+  const size_t own = bytes - ((kept_V || V_kept) ? w.v_elems * sizeof(float) : 0) - (U_kept ? w.u_elems * sizeof(float) : 0);
   float *scratch = (float *)device_alloc(own);
   if (!scratch) {
     if (kept_V) device_free(kept_V);
     if (U_for_dgrad) device_free(U_for_dgrad);
     if (U_kept) device_free(U_kept);
+    if (V_kept) device_free(V_kept);
+    if (dM_for_wgrad) device_free(dM_for_wgrad);
     if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
   float *next = scratch;
   float *U = U_kept ? U_kept : next;
   if (!U_kept) next += w.u_elems;
-  float *V = kept_V ? kept_V : next;
-  if (!kept_V) next += w.v_elems;
+  float *V = kept_V ? kept_V : V_kept ? V_kept : next;
+  if (!kept_V && !V_kept) next += w.v_elems;
   float *Mt = next;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
-  const dim3 fgrid(cdiv(d->K * d->C, 256)), igrid(cdiv(w.Tp, 256), w.Cr), ogrid(cdiv(w.T, 256), w.Mo), block(256);
-  auto transforms_in = [&](auto tile_c) {
-    constexpr int TILE = decltype(tile_c)::value;
-    if (!U_kept)
-      hipLaunchKernelGGL(wino_filter_kernel<TILE>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad, U_for_dgrad);
-    if constexpr (TILE == 4) {
-      if (w.pad_w == 1 && w.in_w % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0) {
-        hipLaunchKernelGGL((wino_input_kernel<4, true>), igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles,
-                           div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
-        return;
-      }
-      if (w.pad_w == 1 && w.in_w % 2 == 0 && (reinterpret_cast<uintptr_t>(in) & 7u) == 0) {
-        hipLaunchKernelGGL((wino_input_kernel<4, true, true>), igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w,
-                           div_tiles, div_tw, w.pad_h, w.pad_w, w.T, w.Tp);
-        return;
-      }
-    }
-    hipLaunchKernelGGL(wino_input_kernel<TILE>, igrid, block, 0, s, in, V, w.Cr, w.in_h, w.in_w, div_tiles, div_tw,
-                       w.pad_h, w.pad_w, w.T, w.Tp);
-  };
-  if (w.tile == 2) transforms_in(IC<2>{}); else transforms_in(IC<4>{});
+  const dim3 fgrid(cdiv(d->K * d->C, 256)), ogrid(cdiv(w.T, 256), w.Mo), block(256);
+  if (!U_kept) {
+    if (w.tile == 2)
+      hipLaunchKernelGGL(wino_filter_kernel<2>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad, U_for_dgrad);
+    else
+      hipLaunchKernelGGL(wino_filter_kernel<4>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad, U_for_dgrad);
+  }
+  if (!V_kept)
+    launch_wino_input(w.tile, in, V, dM_for_wgrad, w.Cr, w.in_h, w.in_w, w.pad_h, w.pad_w, div_tiles, div_tw, w.T, w.Tp,
+                      s);
   with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     const Geometry g = make_geometry(w.Mo, w.Tp, w.Cr, BM, BN, 1, BK);
@@ -1232,6 +1290,13 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
                        div_tiles, div_tw, w.T, w.Tp, rows_vec);
   device_free(scratch);
   if (U_kept) device_free(U_kept);
+  if (V_kept) device_free(V_kept);
+  if (dM_for_wgrad) {
+    d->kept_dy_stream = s;
+    d->kept_dy_tile = 4;
+    d->kept_dy_for = 2;
+    keep_set(&d->kept_dy, dM_for_wgrad, in, (size_t)d->N * d->K * d->P * d->Q * sizeof(float));
+  }
   if (kept_V) {
     d->kept_stream = s;
     d->kept_tile = w.tile;
@@ -1254,43 +1319,48 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
   float *kept_V = nullptr;
   if (d->kept_tile == w.tile && d->kept_stream == s && keeping_transformed_input())
     kept_V = (float *)keep_take(&d->kept_v, x);
+  // dy: grad-data may have left grad-filter's transform of it, or will want its own
+  float *dM_kept = nullptr, *V_for_dgrad = nullptr;
+  if (w.tile == 4 && dy_transforms_shareable(d) && keeping_transformed_input()) {
+    if (d->kept_dy_for == 2 && d->kept_dy_tile == 4 && d->kept_dy_stream == s)
+      dM_kept = (float *)keep_take(&d->kept_dy, dy);
+    if (!dM_kept && d->grad_data_tile == 4) V_for_dgrad = (float *)device_alloc(w.m_elems * sizeof(float));
+  }
   const int KC = d->K * d->C;
   const int bk = stage_depth(plan.bm, plan.bn);
   const Geometry g = make_geometry(d->K, d->C, w.Tp, plan.bm, plan.bn, plan.splits, bk);
   const size_t du_elems = (size_t)g.splits * w.positions * KC;
-  const size_t bytes = ((kept_V ? 0 : w.v_elems) + w.m_elems + du_elems) * sizeof(float);
+  const size_t bytes = ((kept_V ? 0 : w.v_elems) + (dM_kept ? 0 : w.m_elems) + du_elems) * sizeof(float);
   float *scratch = (float *)device_alloc(bytes);
   if (!scratch) {
     if (kept_V) device_free(kept_V);
+    if (dM_kept) device_free(dM_kept);
+    if (V_for_dgrad) device_free(V_for_dgrad);
     if (memorytoSaving) *memorytoSaving = shortfall(bytes);
     return 0;
   }
-  float *V = kept_V ? kept_V : scratch, *dM = kept_V ? scratch : scratch + w.v_elems, *dU = dM + w.m_elems;
+  float *next = scratch;
+  float *V = kept_V ? kept_V : next;
+  if (!kept_V) next += w.v_elems;
+  float *dM = dM_kept ? dM_kept : next;
+  if (!dM_kept) next += w.m_elems;
+  float *dU = next;
   const FastDiv div_tiles((uint32_t)(w.TH * w.TW)), div_tw((uint32_t)w.TW);
   const bool rows_vec = d->Q % w.tile == 0 && (reinterpret_cast<uintptr_t>(dy) & (uintptr_t)(4 * w.tile - 1)) == 0;
   const dim3 block(256);
-  auto transforms_in = [&](auto tile_c) {
-    constexpr int TILE = decltype(tile_c)::value;
-    bool row16 = false, halves = false;
-    if constexpr (TILE == 4) {
-      row16 = d->pad_w == 1 && d->W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-      halves = !row16 && d->pad_w == 1 && d->W % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0;
-    }
-    if (kept_V)
-      ;  // V is the forward call's
-    else if (row16)
-      hipLaunchKernelGGL((wino_input_kernel<4, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
-                         div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
-    else if (halves)
-      hipLaunchKernelGGL((wino_input_kernel<4, true, true>), dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H,
-                         d->W, div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
-    else
-      hipLaunchKernelGGL(wino_input_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->C), block, 0, s, x, V, d->C, d->H, d->W,
-                         div_tiles, div_tw, d->pad_h, d->pad_w, w.T, w.Tp);
-    hipLaunchKernelGGL(wino_dy_kernel<TILE>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q,
-                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
-  };
-  if (w.tile == 2) transforms_in(IC<2>{}); else transforms_in(IC<4>{});
+  if (!kept_V)
+    launch_wino_input(w.tile, x, V, nullptr, d->C, d->H, d->W, d->pad_h, d->pad_w, div_tiles, div_tw, w.T, w.Tp, s);
+  if (dM_kept)
+    ;  // dM is grad-data's by-product
+  else if (V_for_dgrad)  // one pass over dy writes grad-data's V (kept) and dM
+    launch_wino_input(4, dy, V_for_dgrad, dM, d->K, d->P, d->Q, 2 - d->pad_h, 2 - d->pad_w, div_tiles, div_tw, w.T, w.Tp,
+                      s);
+  else if (w.tile == 2)
+    hipLaunchKernelGGL(wino_dy_kernel<2>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q, div_tiles,
+                       div_tw, w.T, w.Tp, rows_vec);
+  else
+    hipLaunchKernelGGL(wino_dy_kernel<4>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q, div_tiles,
+                       div_tw, w.T, w.Tp, rows_vec);
   with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
     const Batched<Across4<BM, BK>> al{{dM, (uint32_t)((size_t)d->K * w.Tp * 4), w.Tp, d->K, w.Tp, FastDiv(ONE_SEGMENT), 0},
@@ -1306,6 +1376,13 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
     hipLaunchKernelGGL(wino_dfilter_kernel<4>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
   device_free(scratch);
   if (kept_V) device_free(kept_V);
+  if (dM_kept) device_free(dM_kept);
+  if (V_for_dgrad) {
+    d->kept_dy_stream = s;
+    d->kept_dy_tile = 4;
+    d->kept_dy_for = 1;
+    keep_set(&d->kept_dy, V_for_dgrad, dy, (size_t)d->N * d->K * d->P * d->Q * sizeof(float));
+  }
   return 0;
 }
 

@@ -129,6 +129,11 @@ struct ConvDesc {
   hipStream_t kept_u_stream = nullptr;
   int kept_u_tile = 0;
   int grad_data_tile = 0;    // tile of the last grad-data call that ran in a Winograd form (0: none yet)
+  // grad-data and grad-filter both transform dy; whichever runs first writes the other's
+  // form along with its own and keeps it (kept_dy_for: 1 grad-data's V, 2 grad-filter's dM)
+  void *kept_dy = nullptr;
+  hipStream_t kept_dy_stream = nullptr;
+  int kept_dy_tile = 0, kept_dy_for = 0;
 };
 
 struct PoolDesc {
