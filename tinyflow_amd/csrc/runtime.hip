@@ -315,7 +315,16 @@ uint64_t record_release_fence(Runtime &r) {
   return number;
 }
 
+int drop_all_kept();  // below, with the registry of kept blocks
+static void *device_alloc_once(size_t bytes);
+// Blocks kept for a later call (keep_set) are a convenience, never a reason to fail:
+// when the device has no room, they are given back and the request is tried again.
 void *device_alloc(size_t bytes) {
+  void *p = device_alloc_once(bytes);
+  if (!p && drop_all_kept() > 0) p = device_alloc_once(bytes);
+  return p;
+}
+static void *device_alloc_once(size_t bytes) {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
   r.init();
@@ -586,10 +595,14 @@ void note_write(const void *ptr, size_t bytes) {
     else ++i;
 }
 
-void note_write_everything() {
-  if (kept_count.load(std::memory_order_acquire) == 0) return;
+void note_write_everything() { (void)drop_all_kept(); }
+
+int drop_all_kept() {
+  if (kept_count.load(std::memory_order_acquire) == 0) return 0;
   std::lock_guard<std::mutex> g(kept_mu);
+  const int n = (int)kept.size();
   while (!kept.empty()) drop_at(kept.size() - 1);
+  return n;
 }
 
 bool device_budget_active() {
