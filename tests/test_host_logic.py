@@ -471,6 +471,87 @@ def test_prefetch_points_placed_by_time():
         assert engine_free <= clock(first_use) + 1e-9 or at_floor, (n.name, engine_free, clock(first_use))
 
 
+def test_budget_recomputes_cheap_convolution_outputs_instead_of_moving_them():
+    """plan_schedule with a budget and ``recompute_instead``: of the tensors the budget
+    would send over the link, the convolution outputs that hang on a short chain are
+    recomputed; fewer bytes move, the simulated footprint still fits, a chain holds at
+    most one such value and five evaluations, and without the option (or without a
+    budget) the plan is the old one."""
+    from tinyflow_amd.SwapExecute import plan_schedule
+    from tinyflow_amd.TrainExecute import getcomputelist, swapsgd
+    rng = np.random.RandomState(0)
+    model = models.resnet(rng, [2, 2, 1, 1], 4, image=32, n_class=10, width=8)
+    variables = list(reversed(ad.get_Variable_node_list(model.loss)))
+    topo = swapsgd(ad.find_topo_sort(getcomputelist(variables, ad.gradients(model.loss, variables), 0.1)))
+    forward = set(ad.find_topo_sort([model.loss]))
+    keep = set(n for n in topo if n.isw in (1, 2)) | {model.loss}
+    shapes = {}
+    feed = {model.X: (4, 3, 32, 32), model.y_: (4, 10)}
+    for n in topo:
+        if n in feed:
+            shapes[n] = feed[n]
+        elif n.isw == 1:
+            shapes[n] = tuple(np.shape(dict(model.variables)[n]))
+        else:
+            shapes[n] = tuple(n.op.infer_shape(n, [shapes[i] for i in n.inputs], None))
+    nbytes = lambda n: 4 * int(np.prod(shapes[n]))
+    cheap = lambda n: isinstance(n.op, (ad.BNForwardOp, ad.ActivationForwardOp))
+    conv = lambda n: isinstance(n.op, ad.Convolution2DForwardOp)
+    args = (topo, forward, keep, lambda n: True, 2)
+    common = dict(nbytes_of=nbytes, recomputable=cheap)
+    # the footprint with recomputation only, then a budget a fifth below its peak
+    pos = {n: i for i, n in enumerate(topo)}
+
+    def peak_of(plan, budget_for_lag=0):
+        out, inn, rel, rec = plan
+        live = np.zeros(len(topo) + 1, dtype=np.int64)
+        persistent = sum(nbytes(n) for n in keep)
+        last = {n: max(t for t, ns in rel.items() if n in ns) for n in topo if n not in keep and not n.issgd}
+        for n, l in last.items():
+            live[pos[n]] += nbytes(n)
+            live[l + 1] -= nbytes(n)
+        live = np.cumsum(live)[:len(topo)] + persistent
+        first_rel = {n: min(t for t, ns in rel.items() if n in ns) for n in last}
+        for t, ns in rec.items():
+            for n in ns:
+                live[first_rel[n] + 1:t] -= nbytes(n)
+        in_at = {n: t for t, ns in inn.items() for n in ns}
+        for t, ns in out.items():
+            for n in ns:
+                live[t + 2 + 1:in_at[n]] -= nbytes(n)
+        return int(live.max())
+
+    free = plan_schedule(*args, budget=1 << 40, **common)
+    assert not free[0], "nothing has to move under a huge budget"
+    budget = int(peak_of(free) * 0.8)
+    plain = plan_schedule(*args, budget=budget, **common)
+    hybrid = plan_schedule(*args, budget=budget, recompute_instead=conv, **common)
+    assert plan_schedule(*args, budget=budget, recompute_instead=lambda n: False, **common) == plain
+    moved = lambda plan: sum(nbytes(n) for ns in plan[0].values() for n in ns)
+    rec_of = lambda plan: {n for ns in plan[3].values() for n in ns}
+    assert moved(plain) > 0
+    heavy = {n for n in rec_of(hybrid) if conv(n)}
+    assert heavy and not any(conv(n) for n in rec_of(plain))
+    assert heavy <= {n for ns in plain[0].values() for n in ns}, "only tensors the budget would have moved"
+    assert moved(hybrid) < moved(plain)
+    assert peak_of(hybrid) <= budget
+
+    rec_at = {n: t for t, ns in hybrid[3].items() for n in ns}
+
+    def chain(n):
+        if n not in rec_at:
+            return 0, 0
+        below = [chain(i) for i in n.inputs]
+        return 1 + max(d for d, _ in below), int(conv(n)) + max(h for _, h in below)
+
+    for n, t in rec_at.items():
+        d, h = chain(n)
+        assert (h == 0 and d <= 2) or (h == 1 and d <= 5), (n.name, d, h)
+        for inp in n.inputs:
+            if inp in rec_at:
+                assert rec_at[inp] <= t
+
+
 def test_planner_wire_format_round_trip():
     """schedule_to_wire / schedule_from_wire: the planner's list format
     (reference Scheduler.py:304-331) carries the same schedule as the dicts."""

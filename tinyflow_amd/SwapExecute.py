@@ -139,8 +139,35 @@ class MemoryManager(threading.Thread):
 
 
 def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of=None, budget=None,
-                  recomputable=None, seconds_of=None, copy_seconds_of=None, copy_slack=1.25):
+                  recomputable=None, seconds_of=None, copy_seconds_of=None, copy_slack=1.25,
+                  recompute_instead=None):
     """Static schedule in the manner of vDNN, optionally with recomputation.
+
+    ``recompute_instead(node)`` (used with a budget): forward values that are far cheaper
+    to evaluate again than to move over the host link (a convolution output whose
+    multiply-adds take a fraction of a millisecond against several milliseconds per
+    direction).  The schedule is first planned without them; those of the tensors it
+    would move that qualify, and whose inputs are kept, moved or cheaply recomputable
+    values, are then recomputed instead and the rest is planned again around them (the
+    way Capuchin chooses between its two mechanisms by cost).  A chain of
+    recomputations holds at most one such value and five evaluations.
+    """
+    plan = lambda heavy: _plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of,
+                                        budget, recomputable, seconds_of, copy_seconds_of, copy_slack, heavy)
+    first = plan(frozenset())
+    if budget is None or recompute_instead is None:
+        return first[:4]
+    moved, depth = first[4], first[5]
+    heavy = frozenset(n for n in moved if recompute_instead(n) and n.inputs and
+                      1 + max(depth.get(i, 0) for i in n.inputs) <= 3)
+    return plan(heavy)[:4] if heavy else first[:4]
+
+
+def _plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distance, nbytes_of, budget,
+                   recomputable, seconds_of, copy_seconds_of, copy_slack, heavy_nodes):
+    """One planning pass (see plan_schedule); ``heavy_nodes``: values recomputed although
+    they are not cheap.  Also returns the moved nodes and the chain depth of every
+    recomputed node.
 
     Returns (swap_out, swap_in, release, recompute), each a dict ``trigger index ->
     [node]``: after the node at ``trigger`` has been issued, the listed tensors are
@@ -180,16 +207,18 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
     movable = [n for n in topo_order if n not in keep and not n.issgd]
 
     # which forward values are recomputed (decided in forward order: depth of the chain)
-    depth = {}
+    depth, heavy = {}, {}
     if recomputable is not None:
         for n in movable:
-            if n not in forward_nodes or not recomputable(n) or not n.inputs:
+            is_heavy = n in heavy_nodes
+            if n not in forward_nodes or not (is_heavy or recomputable(n)) or not n.inputs:
                 continue
             if not any(u >= first_backward for u in uses[n]) or not any(u < first_backward for u in uses[n]):
                 continue
             d = 1 + max((depth.get(i, 0) for i in n.inputs), default=0)
-            if d <= 2:
-                depth[n] = d
+            h = int(is_heavy) + max((heavy.get(i, 0) for i in n.inputs), default=0)
+            if (h == 0 and d <= 2) or (h == 1 and d <= 5):
+                depth[n], heavy[n] = d, h
     # recompute triggers, consumers first, so that the extra use of an input is known
     # when the input's own trigger is chosen
     extra = {n: [] for n in topo_order}
@@ -270,7 +299,7 @@ def plan_schedule(topo_order, forward_nodes, keep, min_bytes_of, prefetch_distan
     for n, out_at, in_at in candidates:
         swap_out.setdefault(out_at, []).append(n)
         swap_in.setdefault(in_at, []).append(n)
-    return swap_out, swap_in, release, recompute
+    return swap_out, swap_in, release, recompute, [c[0] for c in candidates], depth
 
 
 def _fit_budget(candidates, pos, last_use, absent, nbytes_of, persistent, budget, steps, lag, forced=()):
@@ -396,6 +425,9 @@ class SwapExecutor(object):
         self.prefetch_distance = prefetch_distance
         self.memory_budget = memory_budget   # bytes the schedule plans for; None: move every candidate
         self.recompute = recompute           # evaluate normalisation / activation outputs again instead of moving them
+        # with ``recompute``: also evaluate again, rather than move, the convolution outputs that the budget
+        # would send over the host link and that cost the device far less than the link (see plan_schedule)
+        self.recompute_convolutions = True
         self.cudaStream = gpu_op.create_cudaStream()
         self.cudnnHandle = gpu_op.create_cudnnHandle(self.cudaStream)
         self.cublasHandle = gpu_op.create_cublasHandle(self.cudaStream)
@@ -530,6 +562,12 @@ class SwapExecutor(object):
                 else self._estimate_seconds
             timing = dict(seconds_of=seconds_of, copy_slack=self.prefetch_slack,
                           copy_seconds_of=lambda n: self.tensors[n].nbytes / self.host_link_bytes_per_second)
+            if again is not None and self.recompute_convolutions:
+                # a convolution output is recomputed rather than moved when that costs the
+                # device less than an eighth of what the round trip costs the link
+                timing["recompute_instead"] = lambda n: (
+                    isinstance(n.op, ad.Convolution2DForwardOp) and
+                    8.0 * self._estimate_seconds(n) < 2.0 * self.tensors[n].nbytes / self.host_link_bytes_per_second)
         self.swap_out_at, self.swap_in_at, self.release_at, self.recompute_at = plan_schedule(
             self.topo_order, self.forward_nodes, keep, big, self.prefetch_distance,
             nbytes_of=lambda n: self.tensors[n].nbytes, budget=self.memory_budget, recomputable=again,
@@ -724,6 +762,12 @@ class SwapExecutor(object):
         input_vals = [self._on_gpu(self.tensors[i], node.inputs) for i in node.inputs]
         out = self._alloc(t.shape, node.name + " (recompute)", node.inputs)
         wanted = node.op.compute(node, input_vals, out, *handles)
+        for _ in range(3):
+            if not wanted:
+                break
+            # no room for the op's scratch (a convolution): make room and run it again
+            self._alloc(((int(wanted) + 3) // 4,), node.name + " scratch", node.inputs).free_gpu()
+            wanted = node.op.compute(node, input_vals, out, *handles)
         if wanted:
             raise MemoryError("%s: %d bytes of device scratch could not be allocated" % (node.name, wanted))
         t.gpu, t.state = out, GPU
