@@ -20,6 +20,7 @@
 
 #include <hip/hip_runtime.h>
 #include <cstdint>
+#include <type_traits>
 
 namespace tf {
 namespace gemm {
@@ -248,6 +249,9 @@ struct Across4 {
   static constexpr int VPT = D / DSTEP;
   static constexpr int EPT = VPT * 4;
   static_assert(VPT >= 1 && VPT * DSTEP == D, "tile shape");
+  // The four consecutive reduction elements a lane fetches stay together in LDS: the
+  // plane is [d][k] (see gemm_kernel), written with one 16-byte store per vector.
+  static constexpr bool kKContig = true;
   const float *base;
   uint32_t bytes;
   int ld, d_extent, k_extent;
@@ -284,12 +288,19 @@ struct Across4 {
   }
   template <int LD>
   __device__ inline void store(const State &st, float (*tile)[LD], const float (&reg)[EPT]) const {
+    static_assert(LD % 4 == 0, "rows of the LDS plane must keep 16-byte alignment");
 #pragma unroll
-    for (int e = 0; e < VPT; ++e)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) tile[st.k_local + i][st.d_first + e * DSTEP] = reg[4 * e + i];
+    for (int e = 0; e < VPT; ++e) {
+      const f32x4v v = {reg[4 * e], reg[4 * e + 1], reg[4 * e + 2], reg[4 * e + 3]};
+      *reinterpret_cast<f32x4v *>(&tile[st.d_first + e * DSTEP][st.k_local]) = v;
+    }
   }
 };
+
+template <class L, class = void>
+struct lds_k_contig : std::false_type {};
+template <class L>
+struct lds_k_contig<L, std::enable_if_t<L::kKContig>> : std::true_type {};
 
 // ---- epilogue: plain row-major store ---------------------------------------------
 // Stores go through a buffer descriptor over this split's output: a row past
@@ -361,9 +372,21 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   static_assert(TM >= 1 && TN >= 1, "tile too small for a 2x2 wave grid");
-  constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
-  __shared__ float As[2][BK][LDA];
-  __shared__ float Bs[2][BK][LDB];
+  // LDS planes.  An operand whose loader fetches along the reduction (kKContig) is kept
+  // as [m][k]: its vectors go to LDS untransposed, and a lane fetches the four
+  // reduction elements of four consecutive MFMAs with one 16-byte read.  For that the
+  // reduction is walked in a permuted order inside every group of eight: MFMA s of the
+  // group takes k = 8g + s from lanes 0..31 and k = 8g + 4 + s from lanes 32..63, for
+  // both operands alike (a sum does not care).  Without such an operand the planes are
+  // [k][m] / [k][n] and the order is the plain one.
+  constexpr bool AKC = lds_k_contig<ALoader>::value, BKC = lds_k_contig<BLoader>::value;
+  constexpr bool PERM = AKC || BKC;
+  static_assert(!PERM || BK % 8 == 0, "groups of eight reduction elements");
+  constexpr int LDK = BK + LDS_PAD;
+  constexpr int LDA = AKC ? LDK : BM + LDS_PAD, ROWS_A = AKC ? BM : BK;
+  constexpr int LDB = BKC ? LDK : BN + LDS_PAD, ROWS_B = BKC ? BN : BK;
+  __shared__ float As[2][ROWS_A][LDA];
+  __shared__ float Bs[2][ROWS_B][LDB];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -432,6 +455,51 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
     // MFMA operands are read from LDS one sub-step ahead of the MFMAs that use
     // them (two register sets), so the LDS latency sits under the previous
     // sub-step's matrix instructions.
+    if constexpr (PERM) {
+      // fragments of a whole group (four MFMA steps) per fetch, one group ahead
+      f32x4v a4[2][TM], b4[2][TN];
+      auto fetch_group = [&](int gi, int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int m = wm * WM + 32 * i + lcol;
+          if constexpr (AKC) {
+            a4[slot][i] = *reinterpret_cast<const f32x4v *>(&As[buf][m][8 * gi + 4 * lrow]);
+          } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) a4[slot][i][s] = As[buf][8 * gi + 4 * lrow + s][m];
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int n = wn * WN + 32 * j + lcol;
+          if constexpr (BKC) {
+            b4[slot][j] = *reinterpret_cast<const f32x4v *>(&Bs[buf][n][8 * gi + 4 * lrow]);
+          } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) b4[slot][j][s] = Bs[buf][8 * gi + 4 * lrow + s][n];
+          }
+        }
+      };
+      fetch_group(0, 0);
+#pragma unroll
+      for (int gi = 0; gi < BK / 8; ++gi) {
+        const int cur = gi & 1, nxt = cur ^ 1;
+        if (gi + 1 < BK / 8) fetch_group(gi + 1, nxt);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[cur][i][s], b4[cur][j][s], acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      al.template store<LDA>(sa, As[buf ^ 1], ra);
+      bl.template store<LDB>(sb, Bs[buf ^ 1], rb);
+      __syncthreads();
+      buf ^= 1;
+      continue;
+    }
     float a[2][TM], b[2][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) a[0][i] = As[buf][lrow][wm * WM + 32 * i + lcol];
@@ -472,7 +540,11 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const ALoader al, const B
     // and slows every workgroup of the XCD down).  Ordering: all stores of the piece
     // have been acknowledged (s_waitcnt 0) before the barrier that precedes the ticket.
     constexpr int SC1 = 16;  // device scope in the cache-policy operand of the buffer instructions
-    __shared__ unsigned is_last;
+    // the flag lives in the first word of the A planes, which nobody reads any more (every
+    // wave has passed the barrier that ended the reduction loop): the two 128 x 128 planes
+    // of [m][k] operands fill a quarter of a CU's LDS to the byte, and four workgroups
+    // per CU are what the kernel is tuned for
+    unsigned &is_last = *reinterpret_cast<unsigned *>(&As[0][0][0]);
     const int fold_tiles = tiles - fold.first_tile;
     const size_t slot = (size_t)blockIdx.y * fold_tiles + fold_tile;
     constexpr uint32_t kPieceBytes = (uint32_t)(BM * BN) * 4u;
