@@ -160,7 +160,12 @@ def _resnet_shallow(bn_mode, later_steps_bound=1e-3):
         for var, g in grad_nodes.items():
             assert _rel_err(ex.value_of(g).asnumpy(), grads_ref[var.name]) <= bound, (step, var.name)
         for arr, var in zip(out[1:], model.variables):
-            if bound > 1e-3:  # the update carries the gradient's deviation: compare in the same norm
+            if step > 0:
+                # The second step starts from parameters that already differ in the last bits, and
+                # this network amplifies that by about a thousand per step (see the Winograd variant
+                # below): the update carries the gradient's deviation, so it is compared in the
+                # gradient's norm and bound, not element by element (an element near zero has no
+                # relative accuracy left).
                 assert _rel_err(arr.asnumpy(), params[var.name]) <= bound, (step, var.name)
             else:
                 _close(arr.asnumpy(), params[var.name], "param %s step %d" % (var.name, step))
