@@ -771,8 +771,8 @@ using IC = std::integral_constant<int, V>;
 // otherwise as large as its eight MFMAs per wave.
 inline int stage_depth(int bm, int bn) { return (bm == 64 && bn == 64) ? 32 : 16; }
 
-// Forward and grad-data run the 64 x 64 tile with 16-deep stages when the reduction is
-// short (at most 512): half the LDS per workgroup lets eight instead of four share a CU,
+// Forward, the 1x1 grad-data and the Winograd products run the 64 x 64 tile with 16-deep
+// stages when the reduction (per k-split) is short (at most 512): half the LDS per workgroup lets eight instead of four share a CU,
 // which covers the prologue and epilogue that dominate such a workgroup's life (measured
 // -4 % on those launches; +6 % on reductions of 1024, which keep 32).  Plans, k-split
 // ranges and fold decisions are made for 32-deep stages either way (their ranges are
@@ -1295,7 +1295,7 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
       const Batched<Across4<BM, BK>> al{{U, u_bytes, w.Cr, w.Mo, w.Cr, FastDiv(ONE_SEGMENT), 0}, (int64_t)w.Mo * w.Cr};
       launch<BM, BN, BK>(al, bl, ep, w.Cr, g, s, w.positions);
     }
-  });
+  }, run_depth(plan.bm, plan.bn, w.Cr));
   const bool rows_vec = w.out_w % w.tile == 0 && (reinterpret_cast<uintptr_t>(out) & (uintptr_t)(4 * w.tile - 1)) == 0;
   if (w.tile == 2)
     hipLaunchKernelGGL(wino_output_kernel<2>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
@@ -1384,7 +1384,7 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
                                       (int64_t)d->C * w.Tp};
     const StoreBatched ep{{dU, d->C, d->K, d->C, (int64_t)w.positions * KC}, (int64_t)KC};
     launch<BM, BN, BK>(al, bl, ep, w.Tp, g, s, w.positions);
-  });
+  }, run_depth(plan.bm, plan.bn, g.k_per_split));
   if (w.tile == 2)
     hipLaunchKernelGGL(wino_dfilter_kernel<2>, dim3(cdiv(KC, 64)), block, 0, s, (const float *)dU, dw, KC, g.splits);
   else
@@ -1420,6 +1420,9 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
   if (p.winograd) {
     // the batched product is the contraction kernel; its flop count is what it
     // executes (16 or 36 products), 2.25x or 4x below the direct form's
+    const int reduction = which == 2 ? make_geometry(p.M, p.N, p.K, p.bm, p.bn, p.splits, stage_depth(p.bm, p.bn)).k_per_split
+                                     : p.K;
+    const int bk = run_depth(p.bm, p.bn, reduction);
     snprintf(name, (size_t)name_len,
              "%s %dx%d s%d | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<%s<%d, %d>>, StoreBatched>",
              p.variant, p.bm, p.bn, p.splits, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk,
