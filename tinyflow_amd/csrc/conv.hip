@@ -23,6 +23,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <cstring>
 #include <cmath>
 #include <type_traits>
 
@@ -1424,9 +1425,9 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
                                      : p.K;
     const int bk = run_depth(p.bm, p.bn, reduction);
     snprintf(name, (size_t)name_len,
-             "%s %dx%d s%d | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d>>, Batched<%s<%d, %d>>, StoreBatched>",
+             "%s %dx%d s%d | gemm_kernel<%d, %d, %d, Batched<%s<%d, %d%s>>, Batched<%s<%d, %d%s>>, StoreBatched>",
              p.variant, p.bm, p.bn, p.splits, p.bm, p.bn, bk, which == 1 ? "Along4" : "Across4", p.bm, bk,
-             which == 2 ? "Across4" : "Along4", p.bn, bk);
+             which == 1 ? "" : ", false", which == 2 ? "Across4" : "Along4", p.bn, bk, which == 2 ? ", false" : "");
     if (flops) {
       WinoShape w;
       wino_shape(d, which == 1, w, which == 2, p.wino_tile);
@@ -1434,13 +1435,15 @@ extern "C" int DLGpuConvolutionDescribeKernel(void ***list, int which, char *nam
     }
     return 0;
   }
+  // Across4 carries its RAGGED flag in the symbol (a profiler prints defaulted arguments too)
   char b_args[32];
   const bool ragged_wgrad = which == 2 && p.b_vec && p.seg != d->P * d->Q;
+  const char *a_flag = strcmp(p.a_loader, "Across4") == 0 ? (ragged_wgrad ? ", true" : ", false") : "";
+  const char *b_flag = strcmp(p.b_loader, "Across4") == 0 ? (ragged_wgrad ? ", true" : ", false") : "";
   if (p.b_mode >= 0) snprintf(b_args, sizeof b_args, "%d, %d, %d", p.bn, bk, p.b_mode);
-  else snprintf(b_args, sizeof b_args, ragged_wgrad ? "%d, %d, true" : "%d, %d", p.bn, bk);
+  else snprintf(b_args, sizeof b_args, "%d, %d%s", p.bn, bk, b_flag);
   snprintf(name, (size_t)name_len, "%s %dx%d s%d | gemm_kernel<%d, %d, %d, %s<%d, %d%s>, %s<%s>, %s>", p.variant,
-           p.bm, p.bn, p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, ragged_wgrad ? ", true" : "", p.b_loader, b_args,
-           p.epilogue);
+           p.bm, p.bn, p.splits, p.bm, p.bn, bk, p.a_loader, p.bm, bk, a_flag, p.b_loader, b_args, p.epilogue);
   if (flops)
     *flops = 2.0 * d->N * d->K * d->C * d->R * d->S * (double)d->P * d->Q;
   return 0;
