@@ -195,6 +195,58 @@ def test_conv_gradients_are_deterministic(rt):
     np.testing.assert_array_equal(outs[0][1], outs[1][1])
 
 
+SCRATCH_CASES = [
+    ((2, 64, 16, 16, 64, 3, 3, "SAME", 1, 1), "0"),     # direct forms: re-laid filter, k-split partials or fold pieces
+    ((1, 64, 8, 8, 1024, 3, 3, "SAME", 1, 1), "0"),     # one tile, long reduction: grad-data splits
+    ((8, 128, 7, 7, 256, 1, 1, "VALID", 1, 1), "0"),    # 1x1
+    ((4, 64, 28, 28, 64, 3, 3, "SAME", 1, 1), "4"),     # Winograd scratch
+]
+
+
+@pytest.mark.parametrize("case,wino", SCRATCH_CASES, ids=lambda c: "x".join(str(v) for v in c) if isinstance(c, tuple) else "w" + str(c))
+def test_conv_reports_all_the_scratch_it_needs(rt, monkeypatch, case, wino):
+    """With no room for scratch an entry point writes the bytes it wants and returns 0
+    (the reference's workspace convention); a caller that then makes exactly that much
+    room must be able to repeat the call, however many blocks the entry point takes,
+    and gets the bits of a call without a limit."""
+    from tinyflow_amd import gpu_op, ndarray
+    monkeypatch.setenv("TINYFLOW_WINOGRAD", wino)
+    N, C, H, W, K, R, S, padding, u, v = case
+    rng = np.random.RandomState(parity.stable_seed(case))
+    x = rng.normal(0, 1, (N, C, H, W)).astype(np.float32)
+    w = rng.normal(0, 0.05, (K, C, R, S)).astype(np.float32)
+    out_shape, lst = gpu_op.convolution_2d_forward_get_out_shape(x.shape, w.shape, "NCHW", padding, u, v)
+    dy = rng.normal(0, 1, out_shape).astype(np.float32)
+    gx, gw, gdy = _gpu(x, rt), _gpu(w, rt), _gpu(dy, rt)
+    outs = [ndarray.empty(sh, rt.ctx) for sh in (out_shape, x.shape, w.shape)]
+    calls = [lambda o: gpu_op.convolution_2d_forward(gx, gw, o, lst, rt.cudnn, rt.stream),
+             lambda o: gpu_op.convolution_backward_data(gx, gdy, gw, o, lst, rt.cudnn, rt.stream),
+             lambda o: gpu_op.convolution_backward_filter(gx, gdy, gw, o, lst, rt.cudnn, rt.stream)]
+    free = []
+    for call, o in zip(calls, outs):
+        assert call(o) == 0
+        free.append(o.asnumpy())
+    in_use = gpu_op.device_memory_stats()[1]
+    needed_scratch = 0
+    try:
+        for call, o, want in zip(calls, outs, free):
+            gpu_op.set_device_memory_limit(0)
+            gpu_op.set_device_memory_limit(max(in_use, 1))     # nothing more can be allocated
+            gpu_op.array_set(o, np.nan, rt.stream)
+            wanted = call(o)
+            if wanted == 0:                                     # this form takes no scratch
+                assert o.asnumpy().tobytes() == want.tobytes()
+                continue
+            needed_scratch += 1
+            gpu_op.set_device_memory_limit(0)
+            gpu_op.set_device_memory_limit(in_use + -(-wanted // 65536) * 65536)   # budgets count in 64 KiB units
+            assert call(o) == 0, "%d bytes were reported, and with that much room the call still finds none" % wanted
+            assert o.asnumpy().tobytes() == want.tobytes()
+    finally:
+        gpu_op.set_device_memory_limit(0)
+    assert needed_scratch > 0 or wino == "0"
+
+
 def _kept_counts():
     import ctypes
     from tinyflow_amd import _base

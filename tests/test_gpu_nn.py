@@ -122,6 +122,40 @@ def test_max_pool_backward_without_scratch_memory(rt, case):
     np.testing.assert_array_equal(got, gdx.asnumpy())
 
 
+@pytest.mark.parametrize("mode", ["pre_activation", "spatial"])
+def test_batch_norm_reports_all_the_scratch_it_needs(rt, mode):
+    """The out-of-memory convention: a call that finds no room writes the bytes it wants
+    and returns 0; a caller that then makes exactly that much room must be able to repeat
+    the call.  Forward needs two statistics blocks (and spatial mode a partial-sum block
+    on top): with room for one and a half of them the report has to cover all of them."""
+    from tinyflow_amd import gpu_op, ndarray
+    shape = (4, 64, 32, 32) if mode == "pre_activation" else (4, 131072, 2, 2)
+    stats = int(np.prod(shape[1:])) if mode == "pre_activation" else shape[1]
+    block = 4 * stats                                   # 256 KiB / 512 KiB: a multiple of the allocator's rounding
+    x = np.random.RandomState(5).normal(0, 1, shape).astype(np.float32)
+    gx, gy = _gpu(x, rt), ndarray.empty(shape, rt.ctx)
+    mean_p, var_p, lst = gpu_op.bn_get_cudnnlist(shape, "NCHW", mode)
+    in_use = gpu_op.device_memory_stats()[1]
+    gpu_op.set_device_memory_limit(in_use + block + block // 2)
+    try:
+        wanted = gpu_op.bn_forward(gx, gy, mode, 0, mean_p, var_p, lst, rt.cudnn, rt.stream)
+        assert wanted >= 2 * block, "only %d bytes reported for two blocks of %d" % (wanted, block)
+        gpu_op.set_device_memory_limit(0)
+        gpu_op.set_device_memory_limit(in_use + wanted)
+        assert gpu_op.bn_forward(gx, gy, mode, 0, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+        y_ref = O.batch_norm_forward(x.astype(np.float64), mode)[0]
+        np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-3, atol=2e-5)
+    finally:
+        gpu_op.set_device_memory_limit(0)
+    # backward consumes (and releases) the statistics of the repeated call
+    dy = np.random.RandomState(6).normal(0, 1, shape).astype(np.float32)
+    gdx = ndarray.empty(shape, rt.ctx)
+    assert gpu_op.bn_backward(gx, _gpu(dy, rt), gdx, mode, mean_p, var_p, lst, rt.cudnn, rt.stream) == 0
+    _, mean, istd = O.batch_norm_forward(x.astype(np.float64), mode)
+    dx_ref = O.batch_norm_backward(x.astype(np.float64), dy.astype(np.float64), mode, mean, istd)
+    np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-3, atol=2e-5 * max(1.0, float(np.abs(dx_ref).max())))
+
+
 @pytest.mark.parametrize("shape", [(64, 256, 14, 14), (3, 5, 7, 9), (128, 100), (7, 1, 33)])
 @pytest.mark.parametrize("mode", ["relu", "sigmoid", "tanh", "softmax"])
 def test_activation(rt, shape, mode):

@@ -397,11 +397,16 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
     device_free(d->saved_istd);
     d->saved_mean = d->saved_istd = nullptr;
   }
+  // Everything this call allocates, which is what it reports when any of it cannot be had:
+  // a caller that makes that much room must be able to repeat the call.
+  const int sp_real_chunks = (d->mode == 0 || numel(input) == 0) ? 0 : cdiv(d->N, cdiv(d->N, sp_chunks(d->N, d->C)));
+  const size_t sp_partial_bytes = (size_t)sp_real_chunks * d->C * 2 * sizeof(double);
+  const size_t all_bytes = 2 * block_bytes(stat_bytes) + (sp_partial_bytes ? block_bytes(sp_partial_bytes) : 0);
   float *mean = (float *)device_alloc(stat_bytes);
   float *istd = mean ? (float *)device_alloc(stat_bytes) : nullptr;
   if (!mean || !istd) {
     if (mean) device_free(mean);
-    if (memorytoSaving) *memorytoSaving = shortfall(stat_bytes);
+    if (memorytoSaving) *memorytoSaving = shortfall(all_bytes);
     return 0;
   }
   *mean_p = d->saved_mean = mean;
@@ -427,15 +432,14 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
   } else {
     const int chunks = sp_chunks(d->N, d->C);
     const int ipc = cdiv(d->N, chunks);
-    const int real_chunks = cdiv(d->N, ipc);
-    const size_t pbytes = (size_t)real_chunks * d->C * 2 * sizeof(double);
-    double *partial = (double *)device_alloc(pbytes);
+    const int real_chunks = sp_real_chunks;
+    double *partial = (double *)device_alloc(sp_partial_bytes);
     if (!partial) {
       device_free(mean);
       device_free(istd);
       *mean_p = d->saved_mean = nullptr;
       *Variance_p = d->saved_istd = nullptr;
-      if (memorytoSaving) *memorytoSaving = shortfall(pbytes);
+      if (memorytoSaving) *memorytoSaving = shortfall(all_bytes);
       return 0;
     }
     const bool vec = d->HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;

@@ -1609,21 +1609,6 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
     return finish(s, "DLGpuConvolutionBackwardData");
   }
 
-  // filter as [(k, r, s)][c]; a 1x1 filter already has that layout
-  const float *wt = (const float *)filter->data;
-  float *wt_scratch = nullptr;
-  if (RS > 1) {
-    const size_t bytes = (size_t)numel(filter) * sizeof(float);
-    wt_scratch = (float *)device_alloc(bytes);
-    if (!wt_scratch) {
-      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
-      return 0;
-    }
-    const int total = (int)numel(filter);
-    hipLaunchKernelGGL(filter_to_krsc_kernel, dim3(min(cdiv(total, 256), num_cus() * 8)), dim3(256), 0, s,
-                       (const float *)filter->data, wt_scratch, d->K, d->C, RS);
-    wt = wt_scratch;
-  }
   const uint32_t w_bytes = (uint32_t)(numel(filter) * 4), dy_bytes = (uint32_t)(numel(doutput) * 4);
   const int PQ = d->P * d->Q;
   // a strided filter larger than 1x1 always runs on the small tile, unsplit
@@ -1631,20 +1616,41 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   const int g_bm = strided_taps ? 64 : plan.bm, g_bn = strided_taps ? 64 : plan.bn;
   Geometry g = make_geometry(M, plan.N, K, g_bm, g_bn, strided_taps ? 1 : plan.splits, stage_depth(g_bm, g_bn));
   plan_fold(g, K, stage_depth(g_bm, g_bn), 1);
+  // Scratch: the re-laid filter, the fold pieces or the k-split partials.  Whichever of them
+  // cannot be had, the call reports all of them, so that a caller who makes that much room
+  // can repeat it.
+  const size_t wt_bytes = RS > 1 ? (size_t)numel(filter) * sizeof(float) : 0;
+  const size_t partial_bytes = g.splits > 1 ? (size_t)g.splits * numel(dinput) * sizeof(float) : 0;
+  const size_t fold_bytes = g.fold_pieces > 1 ? g.fold_scratch_bytes(g_bm, g_bn, 1) : 0;
+  const size_t all_bytes = (wt_bytes ? block_bytes(wt_bytes) : 0) + (partial_bytes ? block_bytes(partial_bytes) : 0) +
+                           (fold_bytes ? block_bytes(fold_bytes) : 0);
+  // filter as [(k, r, s)][c]; a 1x1 filter already has that layout
+  const float *wt = (const float *)filter->data;
+  float *wt_scratch = nullptr;
+  if (wt_bytes) {
+    wt_scratch = (float *)device_alloc(wt_bytes);
+    if (!wt_scratch) {
+      if (memorytoSaving) *memorytoSaving = shortfall(all_bytes);
+      return 0;
+    }
+    const int total = (int)numel(filter);
+    hipLaunchKernelGGL(filter_to_krsc_kernel, dim3(min(cdiv(total, 256), num_cus() * 8)), dim3(256), 0, s,
+                       (const float *)filter->data, wt_scratch, d->K, d->C, RS);
+    wt = wt_scratch;
+  }
   FoldBuffers fb;
   if (const int rc = acquire_fold(g, g_bm, g_bn, 1, s, fb)) {
     if (wt_scratch) device_free(wt_scratch);
-    if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);
+    if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(all_bytes);
     return rc == 1 ? 0 : -1;
   }
   float *partial = nullptr;
-  if (g.splits > 1) {
-    const size_t bytes = (size_t)g.splits * numel(dinput) * sizeof(float);
-    partial = (float *)device_alloc(bytes);
+  if (partial_bytes) {
+    partial = (float *)device_alloc(partial_bytes);
     if (!partial) {
       if (wt_scratch) device_free(wt_scratch);
       release_fold(fb);
-      if (memorytoSaving) *memorytoSaving = shortfall(bytes);
+      if (memorytoSaving) *memorytoSaving = shortfall(all_bytes);
       return 0;
     }
   }

@@ -17,6 +17,7 @@ namespace tf {
 // them (same stream, or cross-stream wait inserted by DLArrayCopyFromTo).
 void *device_alloc(size_t bytes);  // nullptr when the device (or the cap) is exhausted
 void device_free(void *p);
+size_t block_bytes(size_t bytes);  // what a block of that many bytes occupies (the allocator's rounding)
 void *pinned_alloc(size_t bytes);
 void pinned_free(void *p);
 

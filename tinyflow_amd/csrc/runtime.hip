@@ -315,6 +315,8 @@ uint64_t record_release_fence(Runtime &r) {
   return number;
 }
 
+size_t block_bytes(size_t bytes) { return round_size(bytes); }
+
 int drop_all_kept();  // below, with the registry of kept blocks
 static void *device_alloc_once(size_t bytes);
 // Blocks kept for a later call (keep_set) are a convenience, never a reason to fail:
@@ -341,7 +343,10 @@ static void *device_alloc_once(size_t bytes) {
       return ptr;
     }
   }
-  void *ptr = pool_alloc(r.dev, bytes, true, r.dev_limit);
+  // blocks still alive in an arena that an earlier budget left behind count against this one
+  size_t limit = r.dev_limit;
+  if (limit != 0 && r.arena.base) limit = limit > r.arena.used_bytes ? limit - r.arena.used_bytes : 1;
+  void *ptr = pool_alloc(r.dev, bytes, true, limit);
   if (ptr) {
     auto it = r.pool_fence.find(ptr);
     r.block_fence[ptr] = it == r.pool_fence.end() ? Runtime::kNoFence : it->second;
