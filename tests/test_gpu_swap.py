@@ -170,6 +170,35 @@ def test_budget_arena_never_overlaps_and_coalesces():
         gpu_op.set_device_memory_limit(0)
 
 
+def test_a_new_budget_counts_arrays_that_outlive_the_previous_one():
+    """Changing the budget while arrays of the old budget are alive: those arrays count
+    against the new budget until they are freed."""
+    from tinyflow_amd import gpu_op, ndarray
+    ctx = ndarray.gpu(0)
+    base = gpu_op.device_memory_stats()[1]
+    mib = 1 << 20
+    gpu_op.set_device_memory_limit(base + 8 * mib)
+    try:
+        a = ndarray.empty((mib,), ctx)                     # 4 MiB under the first budget
+        assert not isinstance(a, int)
+        gpu_op.array_set(a, 3.0, None)
+        gpu_op.set_device_memory_limit(base + 6 * mib)
+        assert isinstance(ndarray.empty((mib,), ctx), int)  # 4 + 4 MiB do not fit 6
+        small = ndarray.empty((mib // 4,), ctx)            # 4 + 1 MiB do
+        assert not isinstance(small, int)
+        assert gpu_op.device_memory_stats()[1] - base <= 6 * mib
+        assert np.all(a.asnumpy() == 3.0)
+        a.free_gpu()
+        b = ndarray.empty((mib,), ctx)                     # now 1 + 4 MiB
+        assert not isinstance(b, int)
+        assert gpu_op.device_memory_stats()[1] - base <= 6 * mib
+        b.free_gpu()
+        small.free_gpu()
+        assert gpu_op.device_memory_stats()[1] == base
+    finally:
+        gpu_op.set_device_memory_limit(0)
+
+
 def test_planner_lists_drive_the_step_bit_identically():
     """A schedule handed over in the planner's wire format (swap list, release
     list, recomputation list) gives the same bits as the plain executor: the
