@@ -1,8 +1,9 @@
 """Shared yardsticks of the GPU parity tests.
 
 Three measurements are taken for every compared tensor and appended to a report
-that the session writes to ``gpurun_out/parity_report.json`` (read by nobody at run
-time; the per-family figures quoted in the design notes come from it):
+that the session writes as ``parity_report.json`` into the run's output folder (see
+``write_report``; read by nobody at run time; the per-family figures quoted in the
+design notes come from it):
 
   literal   fraction of elements with |got - ref| <= 1e-5 + 1e-3 * |ref| -- the plain
             rtol 1e-3 / atol 1e-5 bar, with no scaling of the absolute term;
@@ -75,7 +76,7 @@ def compare(got, ref64, ref32, family, what, k, assert_ratio=True):
 def write_report(root):
     if not REPORT:
         return
-    out_dir = os.path.join(root, "gpurun_out")
+    out_dir = os.environ.get("TINYFLOW_PARITY_REPORT_DIR") or os.path.join(root, "gpurun_out")
     try:
         os.makedirs(out_dir, exist_ok=True)
         families = {}
