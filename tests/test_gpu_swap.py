@@ -12,6 +12,16 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _no_garbage_from_earlier_tests():
+    """These tests read the allocator's in-use and peak counters: device arrays of an
+    earlier test that are still waiting for the garbage collector would be freed at
+    some point in the middle of a measurement."""
+    import gc
+    gc.collect()
+    yield
+
+
 def _shallow_resnet(batch=16, image=64, width=8):
     from tinyflow_amd import models
     rng = np.random.RandomState(9)

@@ -575,23 +575,29 @@ class SwapExecutor(object):
 
     def _estimate_seconds(self, node):
         """Rough device time of a node for placing prefetches: a launch, the bytes the
-        node touches at 5.5 TB/s, and for a convolution or matrix product its
-        multiply-adds at 90 TFLOP/s.  Only ratios to the copy times matter."""
+        node touches at 6 TB/s, and for a convolution or matrix product its
+        multiply-adds at 100 TFLOP/s (200 for the 3x3 / stride-1 layers, which run in a
+        Winograd form).  These are the rates of the fast end of what the kernels reach:
+        an estimate that is too short puts a prefetch early, which only holds its
+        storage a little longer, while one that is too long lets the device wait for
+        the copy."""
         if node.isw in (1, 2):
             return 0.0
         moved = self.tensors[node].nbytes + sum(self.tensors[i].nbytes for i in node.inputs)
-        seconds = 5e-6 + moved / 5.5e12
-        flops = 0.0
+        seconds = 5e-6 + moved / 6.0e12
+        flops, rate = 0.0, 100e12
         if isinstance(node.op, (ad.Convolution2DForwardOp, ad.Convolution2DBackwardOp)):
             x, w = self.tensors[node.inputs[0]].shape, self.tensors[node.inputs[1]].shape
             y = self.tensors[node].shape if isinstance(node.op, ad.Convolution2DForwardOp) \
                 else self.tensors[node.inputs[2]].shape
             flops = 2.0 * np.prod(y, dtype=np.float64) * w[1] * w[2] * w[3]
+            if w[2] == 3 and w[3] == 3 and getattr(node, "u", 1) == 1 and getattr(node, "v", 1) == 1:
+                rate = 200e12
         elif isinstance(node.op, ad.MatMulOp):
             a = self.tensors[node.inputs[0]].shape
             flops = 2.0 * np.prod(self.tensors[node].shape, dtype=np.float64) * (a[0] if node.matmul_attr_trans_A
                                                                                  else a[1])
-        return seconds + flops / 90e12
+        return seconds + flops / rate
 
     def _alloc(self, shape, what, protect=()):
         """Device array of ``shape``.  When the budget is exhausted: first wait for
