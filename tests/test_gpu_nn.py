@@ -38,7 +38,9 @@ POOL_CASES = [
     ((2, 3, 70, 130), "max", 0, 0, 2, 2, 2, 2),     # several tiles per plane, ragged last tile
     ((2, 3, 33, 67), "max", 1, 1, 2, 2, 3, 3),
     # planes too large to stage whole in LDS: the 16 x 64 tile kernel, ragged last tiles
-    ((2, 2, 150, 130), "max", 0, 0, 2, 2, 2, 2),
+    ((2, 2, 150, 130), "max", 0, 0, 2, 2, 2, 2),      # unpadded 2x2: bands of 50 rows go through the plane kernels
+    ((2, 3, 224, 224), "max", 0, 0, 2, 2, 2, 2),      # VGG-16's first pool: bands of 56 rows
+    ((1, 2, 146, 130), "max", 0, 0, 2, 2, 2, 2),      # 146 = 2 x 73: no even band divides it, the tile kernel
     ((1, 2, 140, 134), "max", 1, 1, 2, 2, 3, 3),
     # windows too large for the one-pass tile kernel: the two-pass kernels
     ((2, 3, 40, 80), "max", 4, 4, 1, 1, 9, 9),      # stride 1: cell kernel

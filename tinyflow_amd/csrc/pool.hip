@@ -533,6 +533,23 @@ bool shape_is(const DLArray *a, int d0, int d1, int d2, int d3) {
   return a->ndim == 4 && a->shape[0] == d0 && a->shape[1] == d1 && a->shape[2] == d2 && a->shape[3] == d3;
 }
 
+// Rows of x that one workgroup of the plane kernels takes: the whole plane when it fits
+// in LDS; for unpadded 2x2 / stride-2 windows, whose row pairs are independent of one
+// another, otherwise the largest even divisor of H whose band fits (a band of x and its
+// rows of y are contiguous in memory, so a band is a plane of fewer rows); 0: no fit.
+int plane_band_rows(const PoolDesc *d) {
+  const auto fits = [&](int rows, int out_rows) {
+    return rows * d->W <= kPlaneMaxFloats && out_rows * d->Q <= kPlaneWindowsPerLane * kPlaneThreads;
+  };
+  if (fits(d->H, d->P)) return d->H;
+  if (!(d->fh == 2 && d->fw == 2 && d->u == 2 && d->v == 2 && d->pad_h == 0 && d->pad_w == 0 && d->H % 2 == 0 &&
+        d->P * 2 == d->H))
+    return 0;
+  for (int rows = d->H - 2; rows >= 2; rows -= 2)
+    if (d->H % rows == 0 && fits(rows, rows / 2)) return rows;
+  return 0;
+}
+
 }  // namespace
 
 extern "C" int DLGpuPooling2DForwardGetOutShape(const int *input_shapes, int *output_shapes, int dataformat,
@@ -593,10 +610,15 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
     return finish(s, "DLGpuPooling2DForward");
   }
   const bool square2 = d->u == 2 && d->v == 2 && d->fh == d->fw && (d->fh == 2 || d->fh == 3);
-  if (d->mode == 0 && square2 && d->H * d->W <= kPlaneMaxFloats) {
-    const int HW = d->H * d->W;
+  const int band = (d->mode == 0 && square2) ? plane_band_rows(d) : 0;
+  if (band > 0) {
+    PoolParams bp = pp;  // a band of rows is a plane of fewer rows
+    bp.H = band;
+    bp.P = band == d->H ? d->P : band / 2;
+    const PoolParams &pp = bp;
+    const int HW = band * d->W;
     const bool vec = HW % 4 == 0 && (reinterpret_cast<uintptr_t>(input->data) & 15u) == 0;
-    const unsigned planes = (unsigned)(d->N * d->C);
+    const unsigned planes = (unsigned)(d->N * d->C * (d->H / band));
     const size_t lds = (size_t)((HW + 3) / 4 * 4) * sizeof(float);
     const float *xp = (const float *)input->data;
     float *yp = (float *)output->data;
@@ -647,12 +669,17 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
     const int tiles_h = cdiv(d->H, kTileH), tiles_w = cdiv(d->W, kTileW);
     const int64_t blocks = (int64_t)d->N * d->C * tiles_h * tiles_w;
     const bool square2 = d->u == 2 && d->v == 2 && d->fh == d->fw && (d->fh == 2 || d->fh == 3);
-    const int HW = d->H * d->W, PQ = d->P * d->Q;
-    if (square2 && HW <= kPlaneMaxFloats && PQ <= kPlaneWindowsPerLane * kPlaneThreads) {
-      // the whole plane fits in LDS: one workgroup per plane, nothing is read twice
+    const int band = square2 ? plane_band_rows(d) : 0;
+    if (band > 0) {
+      // the plane (or a band of its rows) fits in LDS: one workgroup each, nothing is read twice
+      PoolParams bp = pp;
+      bp.H = band;
+      bp.P = band == d->H ? d->P : band / 2;
+      const PoolParams &pp = bp;
+      const int HW = band * d->W;
       const bool vec = HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(input->data) |
                                         reinterpret_cast<uintptr_t>(dinput->data)) & 15u) == 0;
-      const unsigned planes = (unsigned)(d->N * d->C);
+      const unsigned planes = (unsigned)(d->N * d->C * (d->H / band));
       const size_t lds = (size_t)((HW + 3) / 4 * 4) * sizeof(float);
       const float *xp = (const float *)input->data, *gp = (const float *)doutput->data;
       float *dp = (float *)dinput->data;
