@@ -243,6 +243,34 @@ def test_known_upstream_scalar_gives_the_bits_of_the_read_back(monkeypatch, conf
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("config", ["mlp", "lenet5"])
+def test_known_zero_operand_gives_the_bits_of_the_two_operand_add(monkeypatch, config):
+    """The gradient of a bias broadcast hands a ``zeroslike`` tensor to the adjoint of the
+    broadcast's target, which the graph then adds to the real gradient.  The step
+    executor adds the constant 0.0 instead and never fills that tensor; losses,
+    parameters and every gradient must have the bits of the plain evaluation."""
+    from tinyflow_amd import TrainExecute, models
+    runs, skipped = [], []
+    for shortcut in (True, False):
+        if not shortcut:
+            monkeypatch.setattr(TrainExecute, "_known_zeros_compute", lambda node, shapes: None)
+            monkeypatch.setattr(TrainExecute, "_zeros_only_added", lambda topo, shapes, outputs: set())
+        model, X, y = models.build(config)
+        ex = TrainExecute.TrainExecutor(model.loss, 0.01)
+        ex.init_Variable(dict(model.variables))
+        steps = []
+        for _ in range(3):
+            out = ex.run({model.X: X, model.y_: y})
+            grads = [ex.value_of(g).asnumpy().tobytes() for g in ex.Variable_node_grad_list]
+            steps.append([o.asnumpy().tobytes() for o in out] + grads)
+        skipped.append(sum(1 for n in ex.topo_order if n not in ex.node_to_arr_map))
+        runs.append(steps)
+        ex.close()
+    assert runs[0] == runs[1]
+    assert skipped[0] - skipped[1] >= 3   # one zeros tensor per bias is no longer materialised
+
+
+@pytest.mark.gpu
 def test_fused_update_is_bit_identical_to_per_variable_updates():
     """TrainExecutor(fused_update=True) applies every SGD update of the step with one
     multi-tensor launch behind the last node; losses and parameters over three steps

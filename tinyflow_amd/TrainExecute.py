@@ -88,7 +88,11 @@ class TrainExecutor(object):
             fused.update(find_bn_relu_pairs(self.topo_order, {self.targetloss}))
             fused.update(find_add_relu_pairs(self.topo_order, {self.targetloss}, self.node_to_shape_map))
         self.fused_pairs = sum(1 for v in fused.values() if v[0] in ("forward", "add_relu"))
+        unread_zeros = _zeros_only_added(self.topo_order, self.node_to_shape_map,
+                                         set(self.eval_node_list) | {self.targetloss})
         for node in self.topo_order:
+            if node in unread_zeros:
+                continue   # every reader adds it as the constant 0.0: never materialised
             role = fused.get(node)
             if role is not None and role[0] == "skip":
                 continue   # its value is folded into the fused call of its reader
@@ -106,7 +110,8 @@ class TrainExecutor(object):
                 self.node_to_arr_map[node] = arr
                 continue
             assert node.isw not in (1, 2), "no value fed for %s" % node.name
-            input_vals = [self.node_to_arr_map[i] for i in node.inputs]
+            input_vals = [self.node_to_arr_map.get(i) if i in unread_zeros else self.node_to_arr_map[i]
+                          for i in node.inputs]
             if node.issgd and self.fused_update and isinstance(node.op, ad.SgdOp):
                 fused_sgd.append((input_vals[0], input_vals[1], node.learning_rate))
                 continue
@@ -115,7 +120,8 @@ class TrainExecutor(object):
             else:
                 node_val = self._alloc(self.node_to_shape_map[node])
                 self.node_to_arr_map[node] = node_val
-            plan.append((_known_scalar_compute(node, self.node_to_shape_map) or node.op.compute, node, input_vals,
+            plan.append((_known_scalar_compute(node, self.node_to_shape_map)
+                         or _known_zeros_compute(node, self.node_to_shape_map) or node.op.compute, node, input_vals,
                          node_val))
         self._plan = plan
         if fused_sgd:
@@ -296,6 +302,51 @@ def _known_scalar_compute(node, shapes):
         by_const(input_vals[1 - which], constant, output_val, cudaStream)
         return 0
     return compute
+
+
+def _added_zeros_operand(node, shapes):
+    """Index of the operand of an Add node that is a ``zeroslike`` of the other
+    operand's shape, or None."""
+    if not isinstance(node.op, ad.AddOp) or len(node.inputs) != 2:
+        return None
+    for which in (0, 1):
+        z, other = node.inputs[which], node.inputs[1 - which]
+        if isinstance(z.op, ad.ZerosLikeOp) and shapes[z] == shapes[other] and not isinstance(other.op, ad.ZerosLikeOp):
+            return which
+    return None
+
+
+def _known_zeros_compute(node, shapes):
+    """Plan entry for ``x + zeroslike(.)`` of equal shapes, or None.  The reference's
+    broadcast gradient hands a zeros tensor to its second input (autodiff.py, the
+    ``broadcastto`` gradient), which the accumulation of adjoints then adds to the real
+    gradient: a fill and a two-operand add per bias.  Adding the constant 0.0 gives the
+    same bits (x + 0.0 is the same IEEE sum) with one read less and no fill."""
+    which = _added_zeros_operand(node, shapes)
+    if which is None:
+        return None
+
+    def compute(node, input_vals, output_val, cudnnHandle, cublasHandle, cudaStream):
+        gpu_op.matrix_elementwise_add_by_const(input_vals[1 - which], 0.0, output_val, cudaStream)
+        return 0
+    return compute
+
+
+def _zeros_only_added(topo_order, shapes, outputs):
+    """``zeroslike`` nodes all of whose readers are such additions (and that nobody
+    asks for): their value is never needed as an array."""
+    readers = {}
+    for n in topo_order:
+        for inp in n.inputs:
+            readers.setdefault(inp, []).append(n)
+    unread = set()
+    for z in topo_order:
+        if not isinstance(z.op, ad.ZerosLikeOp) or z in outputs or not readers.get(z):
+            continue
+        if all((_added_zeros_operand(r, shapes) is not None and r.inputs[_added_zeros_operand(r, shapes)] is z)
+               for r in readers[z]):
+            unread.add(z)
+    return unread
 
 
 def _fused_compute(kind, bn):
