@@ -615,7 +615,6 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
     PoolParams bp = pp;  // a band of rows is a plane of fewer rows
     bp.H = band;
     bp.P = band == d->H ? d->P : band / 2;
-    const PoolParams &pp = bp;
     const int HW = band * d->W;
     const bool vec = HW % 4 == 0 && (reinterpret_cast<uintptr_t>(input->data) & 15u) == 0;
     const unsigned planes = (unsigned)(d->N * d->C * (d->H / band));
@@ -625,7 +624,7 @@ extern "C" int DLGpuPooling2DForward(const DLArrayHandle input, DLArrayHandle ou
     auto run = [&](auto f_c, auto vec_c) {
       constexpr int F = decltype(f_c)::value;
       constexpr bool VEC = decltype(vec_c)::value;
-      hipLaunchKernelGGL((pool_max_forward_plane_kernel<F, F, VEC>), dim3(planes), dim3(kPlaneThreads), lds, s, xp, yp, pp);
+      hipLaunchKernelGGL((pool_max_forward_plane_kernel<F, F, VEC>), dim3(planes), dim3(kPlaneThreads), lds, s, xp, yp, bp);
     };
     if (d->fh == 3) { if (vec) run(std::integral_constant<int, 3>{}, std::true_type{}); else run(std::integral_constant<int, 3>{}, std::false_type{}); }
     else { if (vec) run(std::integral_constant<int, 2>{}, std::true_type{}); else run(std::integral_constant<int, 2>{}, std::false_type{}); }
@@ -675,7 +674,6 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
       PoolParams bp = pp;
       bp.H = band;
       bp.P = band == d->H ? d->P : band / 2;
-      const PoolParams &pp = bp;
       const int HW = band * d->W;
       const bool vec = HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(input->data) |
                                         reinterpret_cast<uintptr_t>(dinput->data)) & 15u) == 0;
@@ -687,7 +685,7 @@ extern "C" int DLGpuPooling2DBackward(const DLArrayHandle input, const DLArrayHa
         constexpr int F = decltype(f_c)::value;
         constexpr bool VEC = decltype(vec_c)::value;
         hipLaunchKernelGGL((pool_max_backward_plane_kernel<F, F, VEC>), dim3(planes), dim3(kPlaneThreads), lds, s, xp, gp,
-                           dp, pp);
+                           dp, bp);
       };
       if (d->fh == 3) { if (vec) run(std::integral_constant<int, 3>{}, std::true_type{}); else run(std::integral_constant<int, 3>{}, std::false_type{}); }
       else { if (vec) run(std::integral_constant<int, 2>{}, std::true_type{}); else run(std::integral_constant<int, 2>{}, std::false_type{}); }
