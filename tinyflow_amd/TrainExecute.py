@@ -90,6 +90,9 @@ class TrainExecutor(object):
         self.fused_pairs = sum(1 for v in fused.values() if v[0] in ("forward", "add_relu"))
         unread_zeros = _zeros_only_added(self.topo_order, self.node_to_shape_map,
                                          set(self.eval_node_list) | {self.targetloss})
+        for role in fused.values():   # a fused call reads its sources as arrays
+            if len(role) == 3:
+                unread_zeros -= set(role[2])
         for node in self.topo_order:
             if node in unread_zeros:
                 continue   # every reader adds it as the constant 0.0: never materialised
