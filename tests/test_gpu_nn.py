@@ -185,6 +185,7 @@ def test_activation(rt, shape, mode):
 
 
 BN_SHAPES = [(64, 64, 28, 28), (32, 16, 7, 9), (5, 3, 4, 4), (128, 8, 6, 6), (200, 4, 3, 3), (2, 2048, 7, 7),
+             (65, 5, 9, 7), (100, 64, 14, 14), (128, 256, 14, 14),   # 64 < N <= 128: the 128-row form, ragged and full
              (64, 1, 100), (3, 5, 1, 1), (1, 1300, 2, 2), (7, 300, 5, 5),
              (64, 256, 56, 56)]   # the last one: the largest ResNet-50 b64 activation
 
