@@ -393,6 +393,17 @@ int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int count,
                 const float b1, const float b2, const float b1t, const float b2t,
                 const float e, const float learning_rate);
 
+/* No counterpart in the reference, which allocates the tables above with cudaMalloc
+ * and never gives them back (gpu_op.cu:4628-4700): release calls for the index tables
+ * and for the 2 or 4 pointer tables (device blocks and host cell; the cell is set to
+ * NULL), and index tables for whole tensors laid end to end built from the tensors'
+ * element counts instead of from per-parameter arrays (*count receives the total to
+ * pass to DLGpuSgd_o / DLGpuAdam_o).  The tables come from the library's device pool,
+ * so DLGpuGetDeviceMemoryStats and a memory limit see them. */
+int DLGpuGetTensorRunsCudaPointer(const int64_t *sizes, int n_tensors, int *count, void ***result);
+int DLGpuFreeIndexCudaPointer(void ***indexlist);
+int DLGpuFreeNCudaPointer(void ****list, int n_tables);
+
 #ifdef __cplusplus
 }
 #endif

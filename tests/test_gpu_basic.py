@@ -353,7 +353,44 @@ def test_fused_multi_tensor_updates_with_scattered_indices(rt):
     _fused_case(rt, scattered=True)
 
 
-def _fused_case(rt, scattered):
+def test_fused_multi_tensor_updates_from_tensor_sizes(rt):
+    """The same with the tables built from the tensors' element counts."""
+    _fused_case(rt, scattered=False, from_sizes=True)
+
+
+def test_fused_update_tables_are_counted_and_released(rt):
+    """The index and pointer tables come from the device pool and go back to it: the
+    allocator's in-use figure returns to where it started (the reference never frees
+    them, gpu_op.cu:4628-4700).  Tables that describe whole tensors cost a few hundred
+    bytes, not 8 bytes per parameter; a launch with another count than the tables were
+    built for is refused."""
+    from tinyflow_amd import gpu_op
+    sizes = [1 << 20, 3, 1 << 18]
+    w = [_gpu(np.zeros(n, np.float32), rt) for n in sizes]
+    g = [_gpu(np.ones(n, np.float32), rt) for n in sizes]
+    before = gpu_op.device_memory_stats()[1]
+    number, offset = _flat_index_tables(sizes)
+    t1 = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(np.array(number, np.int32), np.array(offset, np.int32),
+                                                         len(number))
+    t2, count = gpu_op.get_tensor_runs_cuda_pointer(sizes)
+    assert count == sum(sizes)
+    n2 = gpu_op.get_n2_cuda_pointer([a.handle.contents.data for a in w], [a.handle.contents.data for a in g], 3)
+    held = gpu_op.device_memory_stats()[1] - before
+    assert 0 < held < 64 * 1024, held
+    gpu_op.sgd_compute_o(n2, t1, count, 0.5)
+    gpu_op.sgd_compute_o(n2, t2, count, 0.25)
+    with pytest.raises(Exception):
+        gpu_op.sgd_compute_o(n2, t2, count - 1, 0.25)
+    for a in w:
+        np.testing.assert_array_equal(a.asnumpy(), np.full(a.shape, -0.75, np.float32))
+    gpu_op.free_index_cuda_pointer(t1)
+    gpu_op.free_index_cuda_pointer(t2)
+    gpu_op.free_n_cuda_pointer(n2, 2)
+    assert gpu_op.device_memory_stats()[1] == before
+    gpu_op.free_index_cuda_pointer(t1)   # a released cell is null: nothing happens
+
+
+def _fused_case(rt, scattered, from_sizes=False):
     from tinyflow_amd import gpu_op
     # several pieces per tensor (a piece is 4096 elements), odd sizes, one-element tensors
     shapes = [(64, 3, 3, 3), (10,), (1,), (129, 7), (2, 2), (5000, 3), (4096,), (3, 4099)]
@@ -364,7 +401,10 @@ def _fused_case(rt, scattered):
         order = np.random.RandomState(31).permutation(count)
         number, offset = [number[i] for i in order], [offset[i] for i in order]
         tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, count)
-    else:   # numpy tables, as the step executor passes them
+    elif from_sizes:   # as the step executor builds them
+        tables, total = gpu_op.get_tensor_runs_cuda_pointer(sizes)
+        assert total == count
+    else:   # numpy tables
         tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(np.array(number, np.int32), np.array(offset, np.int64),
                                                                  count)
 
@@ -397,6 +437,9 @@ def _fused_case(rt, scattered):
     for name, one, two in (("m", m1, m2), ("v", v1, v2), ("w", w1, w2)):
         for a, b in zip(one, two):
             np.testing.assert_allclose(a.asnumpy(), b.asnumpy(), rtol=2e-7, atol=1e-7, err_msg=name)
+    gpu_op.free_index_cuda_pointer(tables)
+    gpu_op.free_n_cuda_pointer(n2, 2)
+    gpu_op.free_n_cuda_pointer(n4, 4)
 
 
 @pytest.mark.parametrize("shape", [(128, 10), (32, 1000), (7, 3)])

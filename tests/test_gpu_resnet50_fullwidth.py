@@ -10,12 +10,13 @@ eligible 3x3 convolution, grad-data and grad-filter -- the form the planner take
 for all four 3x3 stages at batch 64.
 
 Checked: the loss within rtol 1e-4 of the float64 oracle; every parameter gradient
-in relative L2 within max(5e-2, 3 x the float32 CPU oracle's own distance from the
-float64 one).  A 50-layer batch-normalised stack at batch 8 amplifies rounding (a
-statistic over 8 samples can have near-zero variance), so the float32 CPU oracle
-itself sits 1e-3 ... 1e-1 from float64 in the early layers: the bound is what "as
-close as a numpy fp32 executor" means for this network.  The distances are
-recorded per tensor (tests/parity.py).
+in relative L2 within 3 x the float32 CPU oracle's own distance from the float64
+one + 1e-4 (no other floor).  A 50-layer batch-normalised stack at batch 8 amplifies
+rounding (a statistic over 8 samples can have near-zero variance), so the float32
+CPU oracle itself sits 1e-3 ... 1e-1 from float64 in the early layers: the bound is
+what "as close as a numpy fp32 executor" means for this network.  The distances are
+recorded per tensor (tests/parity.py).  tests/test_gpu_resnet50_b64.py runs the same
+comparison at the benchmark's batch of 64, where the stack is well conditioned.
 """
 import ctypes
 
@@ -87,15 +88,15 @@ def test_resnet50_full_width_step_matches_oracle(monkeypatch, winograd):
         worst = max(worst, err)
         parity.compare(got, grads64[var.name], grads32[var.name], family + ", gradients", var.name, 3.0,
                        assert_ratio=False)
-        assert err <= max(5e-2, 3 * cpu_gap), "gradient of %s: relative L2 %.3g, fp32 CPU oracle %.3g" % (
+        assert err <= 3 * cpu_gap + 1e-4, "gradient of %s: relative L2 %.3g, fp32 CPU oracle %.3g" % (
             var.name, err, cpu_gap)
     for arr, var in zip(out[1:], model.variables):
         parity.compare(arr.asnumpy(), new64[var.name], new32[var.name], family + ", updated parameters", var.name,
                        3.0, assert_ratio=False)
         # the update itself (new - old = -lr * gradient) in the gradient's norm and bound
         old = model.variables[var].astype(np.float64)
-        bound = max(5e-2, 3 * _rel(grads32[var.name], grads64[var.name]))
-        assert _rel(arr.asnumpy().astype(np.float64) - old, new64[var.name] - old) <= bound + 1e-3, var.name
+        bound = 3 * _rel(new32[var.name].astype(np.float64) - old, new64[var.name] - old) + 1e-4
+        assert _rel(arr.asnumpy().astype(np.float64) - old, new64[var.name] - old) <= bound, var.name
     print("winograd=%s: %d of %d conv launches in a Winograd form, loss %.6f (oracle %.6f), worst gradient "
           "relative L2 %.2e" % (winograd, n_wino, len(forms), float(loss[0]), float(loss64[0]), worst))
     ex.close()

@@ -14,7 +14,14 @@ rounding by up to 316x per layer, and ReLU kinks turn that into discrete changes
 the float32 evaluation of the oracle itself then misses the float64 one by far more
 than 1e-3.  For the ResNet case the bound is therefore calibrated per tensor:
 the GPU tensor's relative L2 distance from the float64 oracle must stay within
-the larger of 5e-2 and 3x the float32 oracle's own distance from the float64 oracle.
+3x the float32 oracle's own distance from the float64 oracle + 1e-4 for at least 19 of
+every 20 tensors of a step, and within 3x the largest such distance of the step + 1e-4
+for every tensor.  The second clause is for a decision that flips: in this reduced
+network the last stage is 16 samples x 2 x 2 pixels, so one ReLU that the GPU evaluation
+takes the other way than float64 does (its input lies within rounding of zero) moves
+the gradient of the layer right below it by 1e-2 while the fp32 CPU evaluation, which
+happened to round the other way, sits at 2e-4 there; every layer further down is
+already that far from float64 in both.  There is no constant floor.
 (Measured on the 16-block network: GPU and float32 oracle each sit 1e-2 .. 9e-2 from
 float64, usually 1e-5 from each other, and now and then 1e-2 apart when a single
 ReLU / max-pool decision flips in one of them; a wiring error is O(1).)  The
@@ -92,10 +99,15 @@ def _run_steps(config, lr, steps, build_kw, oracle_kw, calibrated=False, k=K_STE
             continue
         bound = max(1e-3, 4 * _rel_err(loss32, loss_ref))
         assert _rel_err(out[0].asnumpy(), loss_ref) <= bound, "%s step %d loss" % (config, step)
+        gaps = {name: _rel_err(grads32[name], grads_ref[name]) for name in names}
+        errs = {name: _rel_err(got_grads[name], grads_ref[name]) for name in names}
+        step_gap = max(gaps.values())
+        beyond_own = [name for name in names if errs[name] > 3 * gaps[name] + 1e-4]
         for name in names:
-            bound = max(5e-2, 3 * _rel_err(grads32[name], grads_ref[name]))
-            err = _rel_err(got_grads[name], grads_ref[name])
-            assert err <= bound, "%s step %d grad %s: %.3g > %.3g" % (config, step, name, err, bound)
+            assert errs[name] <= 3 * step_gap + 1e-4, "%s step %d grad %s: %.3g > 3 x %.3g (the step's largest " \
+                "fp32 CPU distance) + 1e-4" % (config, step, name, errs[name], step_gap)
+        assert len(beyond_own) <= len(names) // 20, "%s step %d: gradients beyond 3 x their own fp32 CPU distance: %s" % (
+            config, step, ", ".join("%s %.3g > 3 x %.3g" % (n, errs[n], gaps[n]) for n in beyond_own))
         # continue from the GPU's own parameters so that step 2 compares like with like
         params = {name: got_params[name].astype(np.float64) for name in names}
     return ex

@@ -127,6 +127,9 @@ class TrainExecutor(object):
                          or _known_zeros_compute(node, self.node_to_shape_map) or node.op.compute, node, input_vals,
                          node_val))
         self._plan = plan
+        if self._fused_sgd is not None:
+            self._fused_sgd.close()
+            self._fused_sgd = None
         if fused_sgd:
             self._fused_sgd = _FusedSgd(fused_sgd)
         self.isfirstrun = 1
@@ -163,11 +166,15 @@ class TrainExecutor(object):
         """Gives the stream and the two handles back to the library (waits for the
         stream first).  The library orders copies and storage reuse against every
         stream that has run kernels, so an executor that is done should not leave
-        its stream registered.  Arrays already returned stay valid."""
+        its stream registered; the fused update's device tables go back to the pool.
+        Arrays already returned stay valid."""
         if self.cudaStream is None:
             return
         stream, self.cudaStream = self.cudaStream, None
         self._plan = None
+        if self._fused_sgd is not None:
+            self._fused_sgd.close()
+            self._fused_sgd = None
         gpu_op.destroy_cudnnHandle(self.cudnnHandle)
         gpu_op.destroy_cublasHandle(self.cublasHandle)
         gpu_op.destroy_cudaStream(stream)
@@ -194,17 +201,23 @@ class _FusedSgd(object):
         sizes = [int(np.prod(w.shape)) for w, _ in self.arrays]
         for (w, g), n in zip(self.arrays, sizes):
             assert int(np.prod(g.shape)) == n, "gradient and parameter sizes differ"
-        self.count = int(sum(sizes))
-        assert self.count < 2 ** 31
-        number = np.repeat(np.arange(len(sizes), dtype=np.int32), sizes)
-        starts = np.cumsum([0] + sizes[:-1])
-        offset = (np.arange(self.count, dtype=np.int64) - np.repeat(starts, sizes)).astype(np.int32)
-        self.tables = gpu_op.get_index_to_VaribaleNumber_cuda_pointer(number, offset, self.count)
+        assert sum(sizes) < 2 ** 31
+        # whole tensors end to end: the tables are built from the sizes, not from
+        # per-parameter (tensor, offset) arrays
+        self.tables, self.count = gpu_op.get_tensor_runs_cuda_pointer(sizes)
         self.pointers = gpu_op.get_n2_cuda_pointer([w.handle.contents.data for w, _ in self.arrays],
                                                    [g.handle.contents.data for _, g in self.arrays], len(sizes))
 
     def apply(self):
         gpu_op.sgd_compute_o(self.pointers, self.tables, self.count, self.learning_rate)
+
+    def close(self):
+        """Gives the device tables back (waits for the last update that reads them)."""
+        if self.tables is not None:
+            gpu_op.free_index_cuda_pointer(self.tables)
+            gpu_op.free_n_cuda_pointer(self.pointers, 2)
+            self.tables = self.pointers = None
+            self.arrays = []
 
 
 def find_bn_relu_pairs(topo_order, outputs):

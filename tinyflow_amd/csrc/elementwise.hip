@@ -152,6 +152,7 @@ struct RunTable {
   RunPiece *pieces = nullptr;  // device
   int n_pieces = 0;
   int count = 0;               // parameters covered (must equal the launch's count)
+  bool tables_are_dummies = false;  // the per-element tables behind this key were never uploaded
 };
 std::mutex run_mu;
 std::unordered_map<const void *, RunTable> run_tables;  // keyed by the device `number` table
@@ -201,13 +202,16 @@ struct MultiAdam {
   }
 };
 
-// Run table of the launch whose tables start at `number_table`, if its host arrays were runs.
-bool find_run_table(const void *number_table, int count, RunTable &out) {
+// Run table of the launch whose tables start at `number_table`, if its host arrays were
+// runs: 1 found, 0 none (use the indexed kernel), -1 the tables exist only as runs and
+// the launch's count is not the one they were built for.
+int find_run_table(const void *number_table, int count, RunTable &out) {
   std::lock_guard<std::mutex> g(run_mu);
   auto it = run_tables.find(number_table);
-  if (it == run_tables.end() || it->second.count != count || it->second.n_pieces == 0) return false;
+  if (it == run_tables.end()) return 0;
+  if (it->second.count != count || it->second.n_pieces == 0) return it->second.tables_are_dummies ? -1 : 0;
   out = it->second;
-  return true;
+  return 1;
 }
 
 }  // namespace
@@ -393,69 +397,177 @@ extern "C" int DLGpuAdam(DLArrayHandle w, const DLArrayHandle m, const DLArrayHa
 }
 
 // ---- fused multi-tensor SGD --------------------------------------------------
+// Tables of the fused optimizers.  The reference allocates them with cudaMalloc and
+// never gives them back (src/gpu_op.cu:4628-4700); here they come from the pool (so
+// the allocator's statistics and budget see them) and DLGpuFreeIndexCudaPointer /
+// DLGpuFreeNCudaPointer release them.
+
+namespace {
+
+// Records `pieces` under the key `d_number`; false when the device has no room.
+bool publish_runs(const std::vector<RunPiece> &pieces, int count, const void *d_number, bool tables_are_dummies) {
+  RunTable t;
+  t.n_pieces = (int)pieces.size();
+  t.count = count;
+  t.tables_are_dummies = tables_are_dummies;
+  t.pieces = (RunPiece *)device_alloc(pieces.size() * sizeof(RunPiece));
+  if (!t.pieces) return false;
+  if (hipMemcpy(t.pieces, pieces.data(), pieces.size() * sizeof(RunPiece), hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipGetLastError();
+    device_free(t.pieces);
+    return false;
+  }
+  std::lock_guard<std::mutex> g(run_mu);
+  run_tables[d_number] = t;
+  return true;
+}
+
+void append_run(std::vector<RunPiece> &pieces, int tensor, int first_offset, int64_t length) {
+  for (int64_t start = 0; start < length; start += kRunPiece)
+    pieces.push_back(RunPiece{tensor, first_offset + (int)start, (int)std::min<int64_t>(kRunPiece, length - start)});
+}
+
+// The two-pointer result cell of the index tables around device blocks a and b.
+int index_cell(void ***result, void *a, void *b) {
+  *result = (void **)malloc(sizeof(void *) * 2);
+  TF_REQUIRE(*result, "host allocation failed");
+  (*result)[0] = a;
+  (*result)[1] = b;
+  return 0;
+}
+
+}  // namespace
 
 extern "C" int DLGpuGetIndextoVaribaleNumberCudaPointer(int *index_to_number, int *prefix, int count,
                                                         void ***result) {
   TF_REQUIRE(index_to_number && prefix && result && count >= 0, "bad arguments");
-  int *d_number = nullptr, *d_prefix = nullptr;
-  const size_t bytes = sizeof(int) * (size_t)(count > 0 ? count : 1);
-  TF_HIP(hipMalloc((void **)&d_number, bytes));
-  TF_HIP(hipMalloc((void **)&d_prefix, bytes));
-  TF_HIP(hipMemcpy(d_number, index_to_number, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
-  TF_HIP(hipMemcpy(d_prefix, prefix, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
-  *result = (void **)malloc(sizeof(void *) * 2);
-  (*result)[0] = d_number;
-  (*result)[1] = d_prefix;
-  // the same tables as runs of consecutive offsets inside one tensor, cut into pieces
+  // the tables as runs of consecutive offsets inside one tensor, cut into pieces
   std::vector<RunPiece> pieces;
   for (int i = 0; i < count;) {
     int j = i + 1;
     while (j < count && index_to_number[j] == index_to_number[i] && prefix[j] == prefix[i] + (j - i)) ++j;
-    for (int start = i; start < j; start += kRunPiece)
-      pieces.push_back(RunPiece{index_to_number[i], prefix[i] + (start - i), std::min(kRunPiece, j - start)});
+    append_run(pieces, index_to_number[i], prefix[i], j - i);
     i = j;
   }
   // worth it only when the pieces are long on average (scattered indices stay with the indexed kernel)
-  if (!pieces.empty() && (int64_t)pieces.size() * 256 <= (int64_t)count + 256 * 1024) {
-    RunTable t;
-    t.n_pieces = (int)pieces.size();
-    t.count = count;
-    if (hipMalloc((void **)&t.pieces, pieces.size() * sizeof(RunPiece)) == hipSuccess &&
-        hipMemcpy(t.pieces, pieces.data(), pieces.size() * sizeof(RunPiece), hipMemcpyHostToDevice) == hipSuccess) {
-      std::lock_guard<std::mutex> g(run_mu);
-      run_tables[d_number] = t;
-    } else {
-      (void)hipGetLastError();
+  const bool as_runs = !pieces.empty() && (int64_t)pieces.size() * 256 <= (int64_t)count + 256 * 1024;
+  // A launch that finds its run table never reads the per-element tables, so they are
+  // uploaded only for the indexed kernel; the run form keeps two one-word blocks whose
+  // addresses identify the tables.
+  const size_t bytes = as_runs ? sizeof(int) : sizeof(int) * (size_t)(count > 0 ? count : 1);
+  int *d_number = (int *)device_alloc(bytes), *d_prefix = (int *)device_alloc(bytes);
+  if (!d_number || !d_prefix) {
+    if (d_number) device_free(d_number);
+    if (d_prefix) device_free(d_prefix);
+    TF_REQUIRE(false, "no device memory for %zu bytes of index tables", 2 * bytes);
+  }
+  bool published = as_runs && publish_runs(pieces, count, d_number, true);
+  if (as_runs && !published) {
+    device_free(d_number);
+    device_free(d_prefix);
+    TF_REQUIRE(false, "no device memory for the run table");
+  }
+  if (!as_runs && count > 0) {
+    TF_HIP(hipMemcpy(d_number, index_to_number, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
+    TF_HIP(hipMemcpy(d_prefix, prefix, sizeof(int) * (size_t)count, hipMemcpyHostToDevice));
+  }
+  return index_cell(result, d_number, d_prefix);
+}
+
+// No counterpart in the reference: the same index tables for whole tensors laid end to
+// end, built from the tensors' element counts, so that neither the caller nor the
+// library materialises a per-parameter array.  The result is used and released like
+// DLGpuGetIndextoVaribaleNumberCudaPointer's; `*count` receives the parameter total
+// to pass to DLGpuSgd_o / DLGpuAdam_o.
+extern "C" int DLGpuGetTensorRunsCudaPointer(const int64_t *sizes, int n_tensors, int *count, void ***result) {
+  TF_REQUIRE(sizes && result && count && n_tensors >= 0, "bad arguments");
+  int64_t total = 0;
+  std::vector<RunPiece> pieces;
+  for (int t = 0; t < n_tensors; ++t) {
+    TF_REQUIRE(sizes[t] >= 0 && sizes[t] <= INT32_MAX, "tensor %d has a bad size", t);
+    append_run(pieces, t, 0, sizes[t]);
+    total += sizes[t];
+  }
+  TF_REQUIRE(total <= INT32_MAX, "2^31 parameters or more in one fused update");
+  int *d_number = (int *)device_alloc(sizeof(int)), *d_prefix = (int *)device_alloc(sizeof(int));
+  if (!d_number || !d_prefix || (!pieces.empty() && !publish_runs(pieces, (int)total, d_number, true))) {
+    if (d_number) device_free(d_number);
+    if (d_prefix) device_free(d_prefix);
+    TF_REQUIRE(false, "no device memory for the run table");
+  }
+  *count = (int)total;
+  return index_cell(result, d_number, d_prefix);
+}
+
+// No counterpart in the reference (which never releases these tables): gives back the
+// device blocks and the host cell of DLGpuGetIndextoVaribaleNumberCudaPointer /
+// DLGpuGetTensorRunsCudaPointer.  The caller must not use `indexlist` afterwards.
+extern "C" int DLGpuFreeIndexCudaPointer(void ***indexlist) {
+  TF_REQUIRE(indexlist, "bad arguments");
+  if (!*indexlist) return 0;
+  TF_HIP(hipStreamSynchronize(streamless_launch_stream()));  // the last fused update may still read them
+  RunPiece *pieces = nullptr;
+  {
+    std::lock_guard<std::mutex> g(run_mu);
+    auto it = run_tables.find((*indexlist)[0]);
+    if (it != run_tables.end()) {
+      pieces = it->second.pieces;
+      run_tables.erase(it);
     }
   }
+  if (pieces) device_free(pieces);
+  for (int i = 0; i < 2; ++i)
+    if ((*indexlist)[i]) device_free((*indexlist)[i]);
+  free(*indexlist);
+  *indexlist = nullptr;
   return 0;
 }
 
+namespace {
+int pointer_tables(void **const *host, int n_tables, int number, void ****result) {
+  float **dev[4] = {nullptr, nullptr, nullptr, nullptr};
+  const size_t bytes = sizeof(float *) * (size_t)(number > 0 ? number : 1);
+  bool ok = true;
+  for (int i = 0; i < n_tables && ok; ++i) {
+    dev[i] = (float **)device_alloc(bytes);
+    ok = dev[i] && (number == 0 || hipMemcpy(dev[i], host[i], sizeof(float *) * (size_t)number,
+                                             hipMemcpyHostToDevice) == hipSuccess);
+  }
+  void ***cell = ok ? (void ***)malloc(sizeof(void **) * n_tables) : nullptr;
+  if (!cell) {
+    (void)hipGetLastError();
+    for (int i = 0; i < n_tables; ++i)
+      if (dev[i]) device_free(dev[i]);
+    TF_REQUIRE(false, "no memory for %d pointer tables of %d entries", n_tables, number);
+  }
+  for (int i = 0; i < n_tables; ++i) cell[i] = (void **)dev[i];
+  *result = cell;
+  return 0;
+}
+}  // namespace
+
 extern "C" int DLGpuGetN2CudaPointer(void **output, void **g, int number, void ****result) {
   TF_REQUIRE(output && g && result && number >= 0, "bad arguments");
-  float **d_out = nullptr, **d_g = nullptr;
-  const size_t bytes = sizeof(float *) * (size_t)(number > 0 ? number : 1);
-  TF_HIP(hipMalloc((void **)&d_out, bytes));
-  TF_HIP(hipMalloc((void **)&d_g, bytes));
-  TF_HIP(hipMemcpy(d_out, output, sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
-  TF_HIP(hipMemcpy(d_g, g, sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
-  *result = (void ***)malloc(sizeof(void **) * 2);
-  (*result)[0] = (void **)d_out;
-  (*result)[1] = (void **)d_g;
-  return 0;
+  void **host[2] = {output, g};
+  return pointer_tables(host, 2, number, result);
 }
 
 extern "C" int DLGpuGetN4CudaPointer(void **output, void **m, void **v, void **g, int number, void ****result) {
   TF_REQUIRE(output && m && v && g && result && number >= 0, "bad arguments");
   void **host[4] = {output, m, v, g};
-  float **dev[4] = {nullptr, nullptr, nullptr, nullptr};
-  const size_t bytes = sizeof(float *) * (size_t)(number > 0 ? number : 1);
-  for (int i = 0; i < 4; ++i) {
-    TF_HIP(hipMalloc((void **)&dev[i], bytes));
-    TF_HIP(hipMemcpy(dev[i], host[i], sizeof(float *) * (size_t)number, hipMemcpyHostToDevice));
-  }
-  *result = (void ***)malloc(sizeof(void **) * 4);
-  for (int i = 0; i < 4; ++i) (*result)[i] = (void **)dev[i];
+  return pointer_tables(host, 4, number, result);
+}
+
+// No counterpart in the reference: releases the `n_tables` (2 or 4) device pointer
+// tables and the host cell of DLGpuGetN2CudaPointer / DLGpuGetN4CudaPointer.
+extern "C" int DLGpuFreeNCudaPointer(void ****list, int n_tables) {
+  TF_REQUIRE(list && (n_tables == 2 || n_tables == 4), "bad arguments");
+  if (!*list) return 0;
+  TF_HIP(hipStreamSynchronize(streamless_launch_stream()));  // the last fused update may still read them
+  for (int i = 0; i < n_tables; ++i)
+    if ((*list)[i]) device_free((*list)[i]);
+  free(*list);
+  *list = nullptr;
   return 0;
 }
 
@@ -468,7 +580,9 @@ extern "C" int DLGpuAdam_o(void ****n4list, const void ***indexlist, const int c
   // no stream argument: ordered against all streams that run kernels
   hipStream_t s = streamless_launch_stream();
   RunTable runs;
-  if (find_run_table((*indexlist)[0], count, runs)) {
+  const int found = find_run_table((*indexlist)[0], count, runs);
+  TF_REQUIRE(found >= 0, "count %d is not the count the index tables were built for", count);
+  if (found) {
     hipLaunchKernelGGL((multi_tensor_kernel<4, MultiAdam>), dim3(runs.n_pieces), dim3(kThreads), 0, s,
                        MultiAdam{b1, b2, b1t, b2t, e, learning_rate}, (float *const *)((*n4list)[0]),
                        (float *const *)((*n4list)[1]), (float *const *)((*n4list)[2]),
@@ -490,7 +604,9 @@ extern "C" int DLGpuSgd_o(void ****n2list, const void ***indexlist, const int co
   // no stream argument: ordered against all streams that run kernels
   hipStream_t s = streamless_launch_stream();
   RunTable runs;
-  if (find_run_table((*indexlist)[0], count, runs)) {
+  const int found = find_run_table((*indexlist)[0], count, runs);
+  TF_REQUIRE(found >= 0, "count %d is not the count the index tables were built for", count);
+  if (found) {
     hipLaunchKernelGGL((multi_tensor_kernel<2, MultiSgd>), dim3(runs.n_pieces), dim3(kThreads), 0, s,
                        MultiSgd{learning_rate}, (float *const *)((*n2list)[0]), (float *const *)((*n2list)[1]),
                        (float *const *)nullptr, (float *const *)nullptr, (const RunPiece *)runs.pieces);

@@ -409,6 +409,29 @@ def get_index_to_VaribaleNumber_cuda_pointer(index_to_Variable, prefix_list, ind
     return result
 
 
+def get_tensor_runs_cuda_pointer(sizes):
+    """Index tables of the fused optimizers for whole tensors of ``sizes`` elements
+    laid end to end (no counterpart in the reference, which builds per-parameter
+    lists: gpu_op.py:887-945).  Returns (tables, parameter count)."""
+    result = _cell(3)
+    count = ctypes.c_int(0)
+    arr = (ctypes.c_int64 * len(sizes))(*[int(n) for n in sizes])
+    check_call(_LIB.DLGpuGetTensorRunsCudaPointer(arr, ctypes.c_int(len(sizes)), ctypes.byref(count), result))
+    return result, count.value
+
+
+def free_index_cuda_pointer(tables):
+    """Releases the tables of ``get_index_to_VaribaleNumber_cuda_pointer`` /
+    ``get_tensor_runs_cuda_pointer`` (no counterpart in the reference)."""
+    check_call(_LIB.DLGpuFreeIndexCudaPointer(tables))
+
+
+def free_n_cuda_pointer(pointers, n_tables):
+    """Releases the pointer tables of ``get_n2_cuda_pointer`` (n_tables = 2) or
+    ``get_n4_cuda_pointer`` (4) (no counterpart in the reference)."""
+    check_call(_LIB.DLGpuFreeNCudaPointer(pointers, ctypes.c_int(n_tables)))
+
+
 def get_n2_cuda_pointer(output, g, number):
     result = _cell(4)
     check_call(_LIB.DLGpuGetN2CudaPointer(c_array(ctypes.c_void_p, output), c_array(ctypes.c_void_p, g),
