@@ -147,12 +147,18 @@ int DLGpuReduceSumAxisZero(const DLArrayHandle input, DLArrayHandle output);
 /* The same column sums with the same bits, for callers that cannot allocate
  * (code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc).  No counterpart in the reference.  The per-chunk partial sums live
- * in a 2 MiB device array built into the library (one copy per GPU, held until
+ * in a 1.5 MiB device array built into the library (one copy per GPU, held until
  * the process ends) instead of pool memory; no hipMalloc / hipFree / memset is
- * issued.  A shape whose partial sums do not fit returns -1 with a message (2 MiB
- * covers every shape the chunking rule produces for this reduction).  Calls on
+ * issued.  A shape whose partial sums do not fit returns -1 with a message and
+ * launches nothing (on a 256-unit part: chunked sums over more than 131 072
+ * columns; sums that run as one chunk need no scratch and always fit).  Calls on
  * one GPU share the array: calls that overlap on different streams race. */
 int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle input, DLArrayHandle output, void **stream);
+/* The rule behind that limit as pure host arithmetic (no GPU call when cus > 0):
+ * bytes of partial sums a (rows, cols) column sum keeps on a part of `cus` compute
+ * units (0: the current device), and the size of the built-in area.  No
+ * counterpart in the reference. */
+int DLGpuReduceSumAxisZeroNoAllocBytes(int64_t rows, int64_t cols, int cus, int64_t *wanted, int64_t *limit);
 
 /* ref: c_runtime_api.h:110-141, gpu_op.cu:193-219, 1090-1164 */
 int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB,

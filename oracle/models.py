@@ -114,6 +114,22 @@ class Flatten(object):
         return dy.reshape(self.shape)
 
 
+class Dropout(object):
+    """Inverted dropout at rate ``rate`` (reference autodiff.py:1337-1445).  The caller
+    sets ``seed`` before every forward pass: the reference draws a fresh one per
+    evaluation, so a comparison has to hand over the seed the product drew."""
+
+    def __init__(self, rate):
+        self.rate, self.seed = rate, 0
+
+    def forward(self, x, params):
+        y, self.keep = O.dropout_forward(x, self.rate, self.seed)
+        return y
+
+    def backward(self, dy, grads, need_dx=True):
+        return O.dropout_backward(dy, self.keep, self.rate)
+
+
 class Sequential(object):
     def __init__(self, layers):
         self.layers = layers
@@ -164,13 +180,17 @@ def lenet5_layers():
                        Dense("fc3"), Relu(), Dense("fc4"), Relu(), Dense("fc5")])
 
 
-def vgg16_layers():
+def vgg16_layers(dropout=None):
+    """``dropout``: rate of the two dropout layers behind fc6 and fc7 of the reference's
+    model script (pycode/tinyflow/VGG16_test_leo.py:240-247), None for the plain network."""
     layers = []
     for stage, count in enumerate([2, 2, 3, 3, 3], start=1):
         for i in range(1, count + 1):
             layers += [Conv("conv%d_%d" % (stage, i), "SAME", 1), Relu()]
         layers.append(MaxPool(2, 2, 0))
-    layers += [Flatten(), Dense("fc6"), Relu(), Dense("fc7"), Relu(), Dense("fc8")]
+    drop = [] if dropout is None else [Dropout(dropout)]
+    layers += [Flatten(), Dense("fc6"), Relu()] + drop + [Dense("fc7"), Relu()]
+    layers += ([] if dropout is None else [Dropout(dropout)]) + [Dense("fc8")]
     return Sequential(layers)
 
 
@@ -198,6 +218,35 @@ def network(config, bn_mode="pre_activation", image=224):
     raise ValueError(config)
 
 
+def loss_and_gradients(net, params, X, y_onehot, head="softmax_xent"):
+    """Forward + backward of ``net`` under one of the two loss heads.
+
+    ``"softmax_xent"``: mean softmax cross-entropy; the logit gradient is softmax - y
+    WITHOUT the 1/N factor, times the upstream gradient 1 (reference autodiff.py:701-713).
+    ``"cross"``: the head of the reference's ``*_leo`` model scripts
+    (pycode/tinyflow/VGG16_test_leo.py:250-254) on top of the logits: per-feature batch
+    norm over the batch, softmax per instance, loss = sum(-y_ * log(p)) / p.size
+    (reference autodiff.py:2079-2103, 2153-2156), differentiated link by link: cross
+    backward (gpu_op.cu:4568-4573), softmax backward (gpu_op.cu:3521-3531), batch-norm
+    backward, then the network.  Returns (loss, grads, logits)."""
+    logits = net.forward(X, params)
+    grads = {}
+    if head == "softmax_xent":
+        loss = O.softmax_cross_entropy(logits, y_onehot)
+        dlogits = O.softmax_cross_entropy_gradient(logits, y_onehot, 1.0)
+    else:
+        assert head == "cross", head
+        z, mean, istd = O.batch_norm_forward(logits, "pre_activation")
+        p = O.activation_forward(z, "softmax")
+        scale = 1.0 / p.size
+        loss = np.sum(O.cross(p, y_onehot, scale)).reshape(1)
+        dp = O.cross_backward(p, y_onehot, np.ones_like(p), scale)
+        dz = O.activation_backward(z, p, dp, "softmax")
+        dlogits = O.batch_norm_backward(logits, dz, "pre_activation", mean, istd)
+    net.backward(dlogits, grads, need_dx=False)
+    return loss, grads, logits
+
+
 def train_step(net, params, X, y_onehot, lr):
     """One forward + backward + SGD step.
 
@@ -205,26 +254,20 @@ def train_step(net, params, X, y_onehot, lr):
     logit gradient is softmax - y WITHOUT the 1/N factor, times the upstream
     gradient 1 (reference autodiff.py:701-713); new = old - lr * grad
     (reference gpu_op.cu:4600-4605)."""
-    logits = net.forward(X, params)
-    loss = O.softmax_cross_entropy(logits, y_onehot)
-    grads = {}
-    net.backward(O.softmax_cross_entropy_gradient(logits, y_onehot, 1.0), grads, need_dx=False)
+    loss, grads, logits = loss_and_gradients(net, params, X, y_onehot)
     new_params = {k: O.sgd_update(v, grads[k], lr) for k, v in params.items()}
     return loss, grads, new_params, logits
 
 
-def train_step_adam(net, params, moments, X, y_onehot, lr, step, b1=0.9, b2=0.999, e=1e-8):
+def train_step_adam(net, params, moments, X, y_onehot, lr, step, b1=0.9, b2=0.999, e=1e-8, head="softmax_xent"):
     """One forward + backward + Adam step; ``step`` counts from 1.
 
     ``moments`` maps a parameter name to (m, v).  Returns (loss, grads, new_params,
     new_moments).  m, v update: reference gpu_op.cu:4495-4506; parameter update with
     the bias corrections 1 - b1**step, 1 - b2**step: reference gpu_op.cu:4461-4467 and
     TrainExecuteAdam.py:16-21, 196-198 (the powers start at b1, b2 and are multiplied
-    once after every step)."""
-    logits = net.forward(X, params)
-    loss = O.softmax_cross_entropy(logits, y_onehot)
-    grads = {}
-    net.backward(O.softmax_cross_entropy_gradient(logits, y_onehot, 1.0), grads, need_dx=False)
+    once after every step).  ``head``: see ``loss_and_gradients``."""
+    loss, grads, _ = loss_and_gradients(net, params, X, y_onehot, head)
     new_params, new_moments = {}, {}
     for k, w in params.items():
         m, v = O.adam_mv(moments[k][0], moments[k][1], grads[k], b1, b2)
@@ -236,20 +279,7 @@ def train_step_adam(net, params, moments, X, y_onehot, lr, step, b1=0.9, b2=0.99
 def train_step_cross_head(net, params, X, y_onehot, lr):
     """One forward + backward + SGD step with the loss head of the reference's
     ``*_leo`` model scripts (pycode/tinyflow/VGG16_test_leo.py:250-254) on top of
-    ``net``'s logits: per-feature batch norm over the batch, softmax per instance,
-    loss = sum(-y_ * log(p)) / p.size (reference autodiff.py:2079-2103, 2153-2156),
-    differentiated link by link: cross backward (gpu_op.cu:4568-4573), softmax
-    backward (gpu_op.cu:3521-3531), batch-norm backward, then the network.
-    Returns (loss, grads, new_params)."""
-    logits = net.forward(X, params)
-    z, mean, istd = O.batch_norm_forward(logits, "pre_activation")
-    p = O.activation_forward(z, "softmax")
-    scale = 1.0 / p.size
-    loss = np.sum(O.cross(p, y_onehot, scale)).reshape(1)
-    dp = O.cross_backward(p, y_onehot, np.ones_like(p), scale)
-    dz = O.activation_backward(z, p, dp, "softmax")
-    dlogits = O.batch_norm_backward(logits, dz, "pre_activation", mean, istd)
-    grads = {}
-    net.backward(dlogits, grads, need_dx=False)
+    ``net``'s logits (see ``loss_and_gradients``).  Returns (loss, grads, new_params)."""
+    loss, grads, _ = loss_and_gradients(net, params, X, y_onehot, "cross")
     new_params = {k: O.sgd_update(v, grads[k], lr) for k, v in params.items()}
     return loss, grads, new_params

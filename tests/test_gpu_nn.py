@@ -162,8 +162,6 @@ def test_batch_norm_reports_all_the_scratch_it_needs(rt, mode):
 @pytest.mark.parametrize("mode", ["relu", "sigmoid", "tanh", "softmax"])
 def test_activation(rt, shape, mode):
     from tinyflow_amd import gpu_op, ndarray
-    if mode == "softmax" and int(np.prod(shape[1:])) > 4096:
-        pytest.skip("softmax instances this large are not a use case")
     rng = np.random.RandomState(22)
     x = rng.normal(0, 2, shape).astype(np.float32)
     x.flat[::5] = 0.0
@@ -179,6 +177,12 @@ def test_activation(rt, shape, mode):
         np.testing.assert_array_equal(gy.asnumpy(), y_ref.astype(np.float32))
         np.testing.assert_array_equal(gdx.asnumpy(), dx_ref.astype(np.float32))
         assert np.all(gdx.asnumpy().flat[::5] == 0)   # mask is x > 0
+    elif mode == "softmax" and int(np.prod(shape[1:])) > 4096:
+        # an instance of 50 176 elements (no model has one, the library takes it): probabilities of 1e-6 ... 1e-3,
+        # so the absolute terms are scaled to the largest value; sums of 50 176 fp32 terms: rtol 1e-4 / 1e-3
+        np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-4, atol=1e-6 * float(y_ref.max()))
+        np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-3, atol=1e-5 * float(np.abs(dx_ref).max()))
+        np.testing.assert_allclose(gy.asnumpy().astype(np.float64).reshape(shape[0], -1).sum(axis=1), 1.0, rtol=1e-5)
     else:
         np.testing.assert_allclose(gy.asnumpy(), y_ref, rtol=1e-5, atol=1e-6)
         np.testing.assert_allclose(gdx.asnumpy(), dx_ref, rtol=1e-4, atol=1e-6)

@@ -400,3 +400,77 @@ def test_cross_entropy_loss_head_matches_oracle(config):
             got = ex.value_of(grad_nodes[[v for v in model.variables if v.name == name][0]]).asnumpy()
             np.testing.assert_allclose(got / scale, grads_ref[name] / scale, rtol=1e-3, atol=5e-5, err_msg=what + " grad")
             _close(arr.asnumpy(), params[name], what + " param")
+
+
+def test_vgg16_model_script_graph_with_adam_matches_oracle():
+    """The reference's VGG-16 model script as written (pycode/tinyflow/VGG16_test_leo.py:196-254):
+    thirteen 3x3 convolutions with ReLU and five max-pools, flatten, dense + ReLU + dropout(0.5)
+    twice, dense, batch norm of the logits, softmax activation, crossEntropy_loss -- stepped by
+    the Adam executor (the reference's live executor appends one Adam node per variable,
+    autodiff.py:2985-2999) -- at reduced width (32x32 images, 64-wide classifier, 10 classes,
+    batch 16) for two steps against the float64 oracle.
+
+    The dropout op draws its seed from Python's ``random`` on every evaluation, as the
+    reference does; the oracle's two dropout layers are handed the seeds the graph's nodes
+    drew in that step (the masks themselves are bit-identical given the seed,
+    tests/test_gpu_nn.py).  Gradients are held, in relative L2 against float64, to 3x the
+    fp32 CPU evaluation's own distance + 1e-4.  The last bias sits in front of the batch
+    norm, so its gradient is zero in exact arithmetic and rounding residue in fp32; Adam
+    turns any such residue into a step of up to lr, in the reference as here, so that one
+    tensor is bounded absolutely (residue below 1e-4 of the largest gradient norm, parameter
+    within lr per step of its start)."""
+    import random
+    from tinyflow_amd import models
+    from tinyflow_amd import autodiff as ad
+    from tinyflow_amd.TrainExecuteAdam import TrainExecutor
+    lr, rate = 0.001, 0.5
+    kw = dict(batch=16, image=32, n_class=10, fc_width=64)
+    model, X, y = models.build("vgg16", head="cross", dropout=rate, **kw)
+    ex = TrainExecutor(model.loss, lr)
+    ex.init_Variable(dict(model.variables))
+    drop_nodes = [n for n in ex.topo_order if isinstance(n.op, ad.FullyDropoutForwardOp)]
+    assert len(drop_nodes) == 2
+    for op_class in (ad.FullyBNForwardOp, ad.CrossOp, ad.ReduceSumOp, ad.AdamOp):
+        assert any(isinstance(n.op, op_class) for n in ex.topo_order), op_class.__name__
+    names = [v.name for v in model.variables]
+    by_name = {v.name: v for v in model.variables}
+    params = {v.name: val.astype(np.float64) for v, val in model.variables.items()}
+    moments = {k: (np.zeros_like(w), np.zeros_like(w)) for k, w in params.items()}
+    net = OM.vgg16_layers(dropout=rate)
+    drop_layers = [layer for layer in net.layers if isinstance(layer, OM.Dropout)]
+    grad_nodes = dict(zip(ex.Variable_node_list, ex.Variable_node_grad_list))
+    X64, y64 = X.astype(np.float64), y.astype(np.float64)
+    for step in (1, 2):
+        random.seed(40 + step)
+        out = ex.run({model.X: X, model.y_: y})
+        for layer, node in zip(drop_layers, drop_nodes):
+            layer.seed = node.seed[0]
+        p32 = {k: v.astype(np.float32) for k, v in params.items()}
+        m32 = {k: (m.astype(np.float32), v.astype(np.float32)) for k, (m, v) in moments.items()}
+        _, grads32, _, _ = OM.train_step_adam(net, p32, m32, X, y, lr, step, head="cross")
+        loss_ref, grads_ref, new_params, new_moments = OM.train_step_adam(net, params, moments, X64, y64, lr, step,
+                                                                          head="cross")
+        _close(out[0].asnumpy(), loss_ref, "step %d loss" % step, rtol=1e-4)
+        largest = max(float(np.linalg.norm(g)) for g in grads_ref.values())
+        for name, arr in zip(names, out[1:1 + len(names)]):
+            what = "VGG-16 model script, step %d, %s" % (step, name)
+            grad = ex.value_of(grad_nodes[by_name[name]]).asnumpy()
+            m, v = (a.asnumpy() for a in ex.moments_of(by_name[name]))
+            if float(np.linalg.norm(grads_ref[name])) < 1e-6 * largest:
+                assert name == "fc8_b", name
+                assert float(np.linalg.norm(grad)) <= 1e-4 * largest, what
+                assert float(np.abs(arr.asnumpy().astype(np.float64) - model.variables[by_name[name]]).max()) \
+                    <= step * lr * 1.001, what
+                continue
+            parity.compare(grad, grads_ref[name], grads32[name], "train step vgg16 model script (reduced), gradients",
+                           what, 3.0, assert_ratio=False)
+            gap, err = _rel_err(grads32[name], grads_ref[name]), _rel_err(grad, grads_ref[name])
+            assert err <= 3 * gap + 1e-4, "%s grad: %.3g > 3 x %.3g + 1e-4" % (what, err, gap)
+            assert _rel_err(m, new_moments[name][0]) <= 3 * gap + 1e-4, what + " m"
+            assert _rel_err(v, new_moments[name][1]) <= 6 * gap + 2e-4, what + " v"
+            assert _rel_err(arr.asnumpy(), new_params[name]) <= 1e-3, what + " param"
+        # continue from the GPU's own state so that the next step compares like with like
+        params = {name: arr.asnumpy().astype(np.float64) for name, arr in zip(names, out[1:1 + len(names)])}
+        moments = {name: tuple(a.asnumpy().astype(np.float64) for a in ex.moments_of(by_name[name]))
+                   for name in names}
+    ex.close()

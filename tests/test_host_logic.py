@@ -58,6 +58,33 @@ def test_streamed_copy_waits_unless_the_stream_orders_its_readers():
     assert f(D2D, 1, 1) == 1 and f(D2D, 0, 1) == 1
 
 
+def test_no_alloc_column_sum_scratch_rule():
+    """The partial sums the column sum keeps in the library's built-in 1.5 MiB area: on a
+    256-unit part every chunked sum of up to 131 072 columns fits, single-chunk sums want
+    nothing, wider chunked sums are refused; a part with more units wants more (the rule
+    aims at four workgroups per unit), so there narrower sums are refused too."""
+    def wanted(rows, cols, cus):
+        w, lim = ctypes.c_int64(-1), ctypes.c_int64(-1)
+        assert _LIB.DLGpuReduceSumAxisZeroNoAllocBytes(ctypes.c_int64(rows), ctypes.c_int64(cols), cus,
+                                                       ctypes.byref(w), ctypes.byref(lim)) == 0
+        assert lim.value == 3 << 19
+        return w.value, lim.value
+    worst = 0
+    for rows in (1, 7, 8, 9, 64, 1000, 100000):
+        for cols in list(range(1, 70)) + [255, 256, 257, 1000, 3000, 4097, 65536, 100000, 131072]:
+            w, lim = wanted(rows, cols, 256)
+            assert w % (4 * cols) == 0 and w // (4 * cols) != 1      # whole chunks; one chunk needs no scratch
+            assert w // (4 * cols) <= max(1, (rows + 7) // 8)       # at least eight rows per chunk
+            assert w <= lim, (rows, cols, w)
+            worst = max(worst, w)
+    assert worst > lim // 2                                          # the bound is not vacuous
+    assert wanted(64, 200000, 256)[0] == 2 * 200000 * 4 > lim        # refused by the entry point
+    assert wanted(8, 200000, 256)[0] == 0                            # eight rows: one chunk
+    assert wanted(64, 300000, 256)[0] == 0                           # wide enough to fill the part unsplit
+    assert wanted(100000, 100000, 512)[0] > lim                      # a larger part splits further
+    assert wanted(0, 5, 256)[0] == 0 and wanted(5, 0, 256)[0] == 0
+
+
 def test_struct_layout_matches_the_abi():
     """DLContext is 8 bytes, DLArray 32 (src/dlarray.h:21-52)."""
     from tinyflow_amd import ndarray

@@ -116,6 +116,26 @@ def test_cross_head_gradients_are_the_derivative_of_its_loss(case):
     _directional_check(OM.train_step_cross_head, net, params, X, y, 1.0, rng)
 
 
+def test_dropout_layer_and_cross_head_under_finite_differences():
+    """A dense stack with the dropout layer of the reference's VGG-16 script under the
+    batch-norm / softmax / cross head: with the seed held fixed the mask is a constant
+    and the step must still be the derivative of its loss."""
+    rng = np.random.RandomState(15)
+    _, params, X, y = _params_for("mlp", rng)
+    net = OM.Sequential([OM.Dense("fc1"), OM.Relu(), OM.Dropout(0.5), OM.Dense("fc2"), OM.Relu(), OM.Dropout(0.25),
+                         OM.Dense("fc3")])
+    for layer, seed in zip([l for l in net.layers if isinstance(l, OM.Dropout)], (3, 77)):
+        layer.seed = seed
+    _directional_check(OM.train_step_cross_head, net, params, X, y, 1.0, rng)
+    kept = net.layers[2].keep
+    assert 0 < kept.sum() < kept.size          # the mask really drops and keeps something
+
+    def adam(net, params, X, y, lr):
+        moments = {k: (np.zeros_like(v), np.zeros_like(v)) for k, v in params.items()}
+        return OM.train_step_adam(net, params, moments, X, y, lr, 1, head="cross")
+    _directional_check(adam, net, params, X, y, 1.0, rng)
+
+
 def test_sgd_and_adam_steps_apply_their_update_rules_to_those_gradients():
     """new = old - lr * grad for SGD; Adam's first step moves every weight by
     lr * sign(grad) up to e (m / (1 - b1) = g, v / (1 - b2) = g^2)."""

@@ -1527,7 +1527,7 @@ extern "C" int DLGpuConvolution2DForward(const DLArrayHandle input, const DLArra
   }
   const int bm = plan.bm, bn = plan.bn;
   Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
-  plan_fold(g, K, stage_depth(bm, bn), 1);
+  if (fold_tickets(s)) plan_fold(g, K, stage_depth(bm, bn), 1);  // no ticket words: the unfolded plan
   FoldBuffers fb;
   if (const int rc = acquire_fold(g, bm, bn, 1, s, fb)) {
     if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);
@@ -1615,7 +1615,7 @@ extern "C" int DLGpuConvolutionBackwardData(const DLArrayHandle input, const DLA
   const bool strided_taps = RS > 1 && !(d->u == 1 && d->v == 1);
   const int g_bm = strided_taps ? 64 : plan.bm, g_bn = strided_taps ? 64 : plan.bn;
   Geometry g = make_geometry(M, plan.N, K, g_bm, g_bn, strided_taps ? 1 : plan.splits, stage_depth(g_bm, g_bn));
-  plan_fold(g, K, stage_depth(g_bm, g_bn), 1);
+  if (fold_tickets(s)) plan_fold(g, K, stage_depth(g_bm, g_bn), 1);  // no ticket words: the unfolded plan
   // Scratch: the re-laid filter, the fold pieces or the k-split partials.  Whichever of them
   // cannot be had, the call reports all of them, so that a caller who makes that much room
   // can repeat it.
@@ -1751,7 +1751,7 @@ extern "C" int DLGpuConvolutionBackwardFilter(const DLArrayHandle input, const D
 
   const int bm = plan.bm, bn = plan.bn;
   Geometry g = make_geometry(M, N, K, bm, bn, plan.splits, stage_depth(bm, bn));
-  plan_fold(g, K, stage_depth(bm, bn), 1);
+  if (fold_tickets(s)) plan_fold(g, K, stage_depth(bm, bn), 1);  // no ticket words: the unfolded plan
   FoldBuffers fb;
   if (const int rc = acquire_fold(g, bm, bn, 1, s, fb)) {
     if (rc == 1 && memorytoSaving) *memorytoSaving = shortfall(fb.bytes);

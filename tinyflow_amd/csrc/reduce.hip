@@ -223,6 +223,25 @@ __global__ __launch_bounds__(kThreads) void zero_kernel(float *out, int n) {
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// How a sum over A rows (and C inner elements) per output is cut into chunks of rows
+// that separate workgroups sum, so that a short output still fills a part of `cus`
+// compute units (4 workgroups per unit are aimed at); the chunks' partial sums
+// (chunks x B floats) are then added in chunk order.  Pure host arithmetic.
+void chunk_rule(int64_t A, int64_t B, int64_t C, int cus, int &chunks, int &rows_per_chunk) {
+  const int target_blocks = cus * 4;
+  chunks = 1;
+  const int64_t blocks_per_chunk = (C == 1) ? (B + kThreads - 1) / kThreads : B;
+  if (blocks_per_chunk < target_blocks) {
+    chunks = (int)((target_blocks + blocks_per_chunk - 1) / blocks_per_chunk);
+    // keep at least 8 rows per chunk (column sums) / 1 row (mid sums)
+    const int64_t max_chunks = (C == 1) ? (A + 7) / 8 : A;
+    if (chunks > max_chunks) chunks = (int)max_chunks;
+    if (chunks < 1) chunks = 1;
+  }
+  rows_per_chunk = (int)((A + chunks - 1) / chunks);
+  chunks = (int)((A + rows_per_chunk - 1) / rows_per_chunk);
+}
+
 // out[b] = sum_{a, c} in[a, b, c]; 0 on success, 1 when scratch is exhausted
 // (then *scratch_bytes holds the size wanted), -1 on launch failure.  A caller
 // that cannot report exhausted scratch passes scratch_bytes == nullptr: the sum
@@ -244,18 +263,9 @@ int reduce_abc(const float *in, float *out, int64_t A, int64_t B, int64_t C, hip
     hipLaunchKernelGGL(zero_kernel, dim3(cdiv(B, kThreads)), dim3(kThreads), 0, s, out, (int)B);
     return finish(s, what);
   }
-  const int target_blocks = num_cus() * 4;
-  int chunks = 1;
-  int64_t blocks_per_chunk = (C == 1) ? (B + kThreads - 1) / kThreads : B;
-  if (blocks_per_chunk < target_blocks) {
-    chunks = (int)((target_blocks + blocks_per_chunk - 1) / blocks_per_chunk);
-    // keep at least 8 rows per chunk (column sums) / 1 row (mid sums)
-    const int64_t max_chunks = (C == 1) ? (A + 7) / 8 : A;
-    if (chunks > max_chunks) chunks = (int)max_chunks;
-    if (chunks < 1) chunks = 1;
-  }
-  int rows_per_chunk = (int)((A + chunks - 1) / chunks);
-  chunks = (int)((A + rows_per_chunk - 1) / rows_per_chunk);
+  const int64_t blocks_per_chunk = (C == 1) ? (B + kThreads - 1) / kThreads : B;
+  int chunks, rows_per_chunk;
+  chunk_rule(A, B, C, num_cus(), chunks, rows_per_chunk);
   float *partial = out;
   if (chunks > 1) {
     const size_t bytes = (size_t)chunks * (size_t)B * sizeof(float);
@@ -315,7 +325,10 @@ extern "C" int DLGpuReduceSumAxisZero(const DLArrayHandle in, DLArrayHandle out)
 // pool memory.  Each device holds its own copy of the array at its own address, so
 // the address is looked up once per device (hipGetSymbolAddress with that device
 // current) and that pointer, never the symbol, is what the kernels receive.
-constexpr size_t kFixedScratchBytes = 2u << 20;
+// 1.5 MiB: on a 256-unit part chunks x columns stays under 256 Ki + columns floats, so
+// every column sum of up to 131 072 columns fits, and so does any sum that runs as one
+// chunk; a wider chunked sum is refused (DLGpuReduceSumAxisZeroNoAllocBytes tells).
+constexpr size_t kFixedScratchBytes = 3u << 19;
 static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
 
 namespace {
@@ -343,6 +356,23 @@ float *fixed_scratch_of_current_device(const char *what) {
   return fixed_ptr[dev];
 }
 }  // namespace
+
+// Pure host arithmetic, no GPU call when cus > 0: the bytes of partial sums the column
+// sum of a (rows, cols) array keeps in the built-in area on a part of `cus` compute
+// units (0: the current device's count), and the size of that area.  The entry point
+// below refuses a shape with *wanted > *limit.
+extern "C" int DLGpuReduceSumAxisZeroNoAllocBytes(int64_t rows, int64_t cols, int cus, int64_t *wanted,
+                                                  int64_t *limit) {
+  TF_REQUIRE(wanted && limit && rows >= 0 && cols >= 0 && cus >= 0, "bad arguments");
+  TF_REQUIRE(rows <= INT32_MAX && cols <= INT32_MAX, "extents of 2^31 or more are not supported");
+  *limit = (int64_t)kFixedScratchBytes;
+  *wanted = 0;
+  if (rows == 0 || cols == 0) return 0;
+  int chunks, rows_per_chunk;
+  chunk_rule(rows, cols, 1, cus > 0 ? cus : num_cus(), chunks, rows_per_chunk);
+  if (chunks > 1) *wanted = (int64_t)chunks * cols * (int64_t)sizeof(float);
+  return 0;
+}
 
 extern "C" int DLGpuReduceSumAxisZeroNoAlloc(const DLArrayHandle in, DLArrayHandle out, void **stream) {
   announce_write(out);

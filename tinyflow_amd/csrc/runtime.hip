@@ -416,16 +416,20 @@ hipStream_t stream_of(void **cell) {
 // itself: kFoldTicketSlots words per stream, zero between launches (the kernels
 // restore the zeros; launches on one stream run one after the other, so they can
 // share the words).  Allocated on first use and cleared by a fill kernel on `s`.
+// Streams made by DLGpuCreatecudaStream keep their words in their record (released
+// with the stream); any other handle -- the null stream, a caller's own stream -- gets
+// words of its own under its handle, so two such streams never count on the same words.
 unsigned *fold_tickets(hipStream_t s) {
   Runtime &r = rt();
   std::lock_guard<std::mutex> g(r.mu);
-  static unsigned *default_stream_tickets = nullptr;
-  unsigned **cell = &default_stream_tickets;
+  static std::unordered_map<hipStream_t, unsigned *> foreign_stream_tickets;
+  unsigned **cell = nullptr;
   for (auto &rec : r.streams)
     if (rec.stream == s) {
       cell = &rec.fold_tickets;
       break;
     }
+  if (!cell) cell = &foreign_stream_tickets[s];
   if (!*cell) {
     void *p = nullptr;
     if (hipMalloc(&p, kFoldTicketSlots * sizeof(unsigned)) != hipSuccess || !p) {

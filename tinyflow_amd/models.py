@@ -127,7 +127,10 @@ def lenet5(rng, batch=64, head="softmax_xent"):
 VGG16_CHANNELS = [(64, 64), (128, 128), (256, 256, 256), (512, 512, 512), (512, 512, 512)]
 
 
-def vgg16(rng, batch=32, image=224, n_class=1000, fc_width=4096):
+def vgg16(rng, batch=32, image=224, n_class=1000, fc_width=4096, head="softmax_xent", dropout=None):
+    """``head="cross"`` with ``dropout=0.5`` is the graph of the reference's model script
+    as written (pycode/tinyflow/VGG16_test_leo.py:196-254): dropout behind fc6 and fc7,
+    batch norm of the logits, softmax activation, ``crossEntropy_loss``."""
     b = _Builder(rng)
     X, y_ = ad.Placeholder("X"), ad.Placeholder("y_")
     h, in_ch = X, 3
@@ -140,9 +143,13 @@ def vgg16(rng, batch=32, image=224, n_class=1000, fc_width=4096):
     h = ad.flatten_op(h)
     flat = in_ch * (image // 32) ** 2
     h = ad.fullyactivation_forward_op(b.dense(h, "fc6", flat, fc_width), "NCHW", "relu")
+    if dropout is not None:
+        h = ad.fullydropout_forward_op(h, "NCHW", dropout)
     h = ad.fullyactivation_forward_op(b.dense(h, "fc7", fc_width, fc_width), "NCHW", "relu")
+    if dropout is not None:
+        h = ad.fullydropout_forward_op(h, "NCHW", dropout)
     h = b.dense(h, "fc8", fc_width, n_class)
-    loss = ad.softmaxcrossentropy_op(h, y_)
+    loss = _loss_head(h, y_, head)
     return Model("vgg16", loss, h, X, y_, b.variables, (batch, 3, image, image), n_class)
 
 
