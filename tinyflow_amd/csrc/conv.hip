@@ -1237,22 +1237,21 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
   if (!wino_shape(d, dgrad, w, false, plan.wino_tile)) return -1;
   const size_t bytes = (w.u_elems + w.v_elems + w.m_elems) * sizeof(float);
   float *kept_V = nullptr;
-  if (!dgrad && d->grad_filter_tile == w.tile && keeping_transformed_input())
+  if (!dgrad && d->grad_filter_tile == w.tile && keeping_transformed_input() && keep_has_room(w.v_elems * sizeof(float)))
     kept_V = (float *)device_alloc(w.v_elems * sizeof(float));  // no room: this call keeps nothing
   // The transformed filter: a forward call also writes the one grad-data will want (a block
   // of its own, valid until anything writes to the filter); grad-data takes that over.
   float *U_for_dgrad = nullptr, *U_kept = nullptr;
   if (dgrad) d->grad_data_tile = w.tile;
-  if (dgrad && d->kept_u_tile == w.tile && d->kept_u_stream == s && keeping_transformed_input())
-    U_kept = (float *)keep_take(&d->kept_u, filter);
-  if (!dgrad && d->grad_data_tile == w.tile && keeping_transformed_input())
+  if (dgrad && keeping_transformed_input()) U_kept = (float *)keep_take(&d->kept_u, filter, s, w.tile);
+  if (!dgrad && d->grad_data_tile == w.tile && keeping_transformed_input() && keep_has_room(w.u_elems * sizeof(float)))
     U_for_dgrad = (float *)device_alloc(w.u_elems * sizeof(float));
   // dy: grad-filter may have left grad-data's transform of it, or will want its own
   float *V_kept = nullptr, *dM_for_wgrad = nullptr;
   if (dgrad && w.tile == 4 && dy_transforms_shareable(d) && keeping_transformed_input()) {
-    if (d->kept_dy_for == 1 && d->kept_dy_tile == 4 && d->kept_dy_stream == s)
-      V_kept = (float *)keep_take(&d->kept_dy, in);
-    if (!V_kept && d->grad_filter_tile == 4) dM_for_wgrad = (float *)device_alloc(w.v_elems * sizeof(float));
+    V_kept = (float *)keep_take(&d->kept_dy, in, s, kKeptDyForDgrad | 4);
+    if (!V_kept && d->grad_filter_tile == 4 && keep_has_room(w.v_elems * sizeof(float)))
+      dM_for_wgrad = (float *)device_alloc(w.v_elems * sizeof(float));
   }
   const size_t own = bytes - ((kept_V || V_kept) ? w.v_elems * sizeof(float) : 0) - (U_kept ? w.u_elems * sizeof(float) : 0);
   float *scratch = (float *)device_alloc(own);
@@ -1307,22 +1306,15 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
   device_free(scratch);
   if (U_kept) device_free(U_kept);
   if (V_kept) device_free(V_kept);
-  if (dM_for_wgrad) {
-    d->kept_dy_stream = s;
-    d->kept_dy_tile = 4;
-    d->kept_dy_for = 2;
-    keep_set(&d->kept_dy, dM_for_wgrad, in, (size_t)d->N * d->K * d->P * d->Q * sizeof(float));
-  }
-  if (kept_V) {
-    d->kept_stream = s;
-    d->kept_tile = w.tile;
-    keep_set(&d->kept_v, kept_V, in, (size_t)d->N * d->C * d->H * d->W * sizeof(float));
-  }
-  if (U_for_dgrad) {
-    d->kept_u_stream = s;
-    d->kept_u_tile = w.tile;
-    keep_set(&d->kept_u, U_for_dgrad, filter, (size_t)d->K * d->C * 9 * sizeof(float));
-  }
+  if (dM_for_wgrad)
+    keep_set(&d->kept_dy, dM_for_wgrad, w.v_elems * sizeof(float), in, (size_t)d->N * d->K * d->P * d->Q * sizeof(float),
+             s, kKeptDyForWgrad | 4);
+  if (kept_V)
+    keep_set(&d->kept_v, kept_V, w.v_elems * sizeof(float), in, (size_t)d->N * d->C * d->H * d->W * sizeof(float), s,
+             w.tile);
+  if (U_for_dgrad)
+    keep_set(&d->kept_u, U_for_dgrad, w.u_elems * sizeof(float), filter, (size_t)d->K * d->C * 9 * sizeof(float), s,
+             w.tile);
   return 0;
 }
 
@@ -1333,14 +1325,13 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
   d->grad_filter_tile = w.tile;
   // V of this step's forward call, if it is still there, belongs to this x, this tile and this stream
   float *kept_V = nullptr;
-  if (d->kept_tile == w.tile && d->kept_stream == s && keeping_transformed_input())
-    kept_V = (float *)keep_take(&d->kept_v, x);
+  if (keeping_transformed_input()) kept_V = (float *)keep_take(&d->kept_v, x, s, w.tile);
   // dy: grad-data may have left grad-filter's transform of it, or will want its own
   float *dM_kept = nullptr, *V_for_dgrad = nullptr;
   if (w.tile == 4 && dy_transforms_shareable(d) && keeping_transformed_input()) {
-    if (d->kept_dy_for == 2 && d->kept_dy_tile == 4 && d->kept_dy_stream == s)
-      dM_kept = (float *)keep_take(&d->kept_dy, dy);
-    if (!dM_kept && d->grad_data_tile == 4) V_for_dgrad = (float *)device_alloc(w.m_elems * sizeof(float));
+    dM_kept = (float *)keep_take(&d->kept_dy, dy, s, kKeptDyForWgrad | 4);
+    if (!dM_kept && d->grad_data_tile == 4 && keep_has_room(w.m_elems * sizeof(float)))
+      V_for_dgrad = (float *)device_alloc(w.m_elems * sizeof(float));
   }
   const int KC = d->K * d->C;
   const int bk = stage_depth(plan.bm, plan.bn);
@@ -1393,12 +1384,9 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
   device_free(scratch);
   if (kept_V) device_free(kept_V);
   if (dM_kept) device_free(dM_kept);
-  if (V_for_dgrad) {
-    d->kept_dy_stream = s;
-    d->kept_dy_tile = 4;
-    d->kept_dy_for = 1;
-    keep_set(&d->kept_dy, V_for_dgrad, dy, (size_t)d->N * d->K * d->P * d->Q * sizeof(float));
-  }
+  if (V_for_dgrad)
+    keep_set(&d->kept_dy, V_for_dgrad, w.m_elems * sizeof(float), dy, (size_t)d->N * d->K * d->P * d->Q * sizeof(float), s,
+             kKeptDyForDgrad | 4);
   return 0;
 }
 

@@ -66,8 +66,14 @@ int num_cus();
 // the arrays it is about to write (or free) before it does anything else, and the
 // registry drops what was derived from them.  All device memory behind this ABI is
 // written through these entry points, which is what makes the rule complete.
-void keep_set(void **slot, void *block, const void *src, size_t src_bytes);  // replaces what the slot held
-void *keep_take(void **slot, const void *src);  // the block if it is still valid for `src` (caller frees), else null
+// What a block is (`tag`: the owner's code for form and tile) and the stream whose work
+// made it live in the registry entry, under its lock; only a call on that stream asking
+// for that tag and that source gets the block.  All kept blocks together are capped at a
+// fraction of the device's memory: ask keep_has_room before allocating one.
+bool keep_has_room(size_t block_bytes);
+void keep_set(void **slot, void *block, size_t block_bytes, const void *src, size_t src_bytes, hipStream_t stream,
+              int tag);  // replaces what the slot held
+void *keep_take(void **slot, const void *src, hipStream_t stream, int tag);  // the block (caller frees), else null
 void note_write(const void *ptr, size_t bytes);
 void note_write_everything();
 bool device_budget_active();  // a device-memory limit is set: keep nothing
@@ -120,22 +126,19 @@ struct ConvDesc {
   int pad_h, pad_w, u, v;
   // Winograd forms: the transformed input V of the last forward call, kept for the
   // grad-filter call of the same step, which needs exactly this array (see keep_set).
+  // (the three kept_* pointers are registry slots: written and read only through
+  // keep_set / keep_take, which hold the block's tile, form and stream under their lock)
   void *kept_v = nullptr;
-  hipStream_t kept_stream = nullptr;
-  int kept_tile = 0;
   int grad_filter_tile = 0;  // tile of the last grad-filter call that ran in a Winograd form (0: none yet)
   // the same for the transformed filter of grad-data (the filter rotated by 180 degrees),
   // which the forward call's filter transform writes along with its own
   void *kept_u = nullptr;
-  hipStream_t kept_u_stream = nullptr;
-  int kept_u_tile = 0;
   int grad_data_tile = 0;    // tile of the last grad-data call that ran in a Winograd form (0: none yet)
   // grad-data and grad-filter both transform dy; whichever runs first writes the other's
-  // form along with its own and keeps it (kept_dy_for: 1 grad-data's V, 2 grad-filter's dM)
+  // form along with its own and keeps it (tag kKeptDyForDgrad: grad-data's V, kKeptDyForWgrad: grad-filter's dM)
   void *kept_dy = nullptr;
-  hipStream_t kept_dy_stream = nullptr;
-  int kept_dy_tile = 0, kept_dy_for = 0;
 };
+constexpr int kKeptDyForDgrad = 0x100, kKeptDyForWgrad = 0x200;  // or-ed with the tile
 
 struct PoolDesc {
   int magic;

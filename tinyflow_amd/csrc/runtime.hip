@@ -421,25 +421,36 @@ hipStream_t stream_of(void **cell) {
 // words of its own under its handle, so two such streams never count on the same words.
 unsigned *fold_tickets(hipStream_t s) {
   Runtime &r = rt();
-  std::lock_guard<std::mutex> g(r.mu);
-  static std::unordered_map<hipStream_t, unsigned *> foreign_stream_tickets;
-  unsigned **cell = nullptr;
-  for (auto &rec : r.streams)
-    if (rec.stream == s) {
-      cell = &rec.fold_tickets;
-      break;
-    }
-  if (!cell) cell = &foreign_stream_tickets[s];
-  if (!*cell) {
-    void *p = nullptr;
-    if (hipMalloc(&p, kFoldTicketSlots * sizeof(unsigned)) != hipSuccess || !p) {
+  auto cell_of = [&]() -> unsigned ** {  // with r.mu held
+    static std::unordered_map<hipStream_t, unsigned *> foreign_stream_tickets;
+    for (auto &rec : r.streams)
+      if (rec.stream == s) return &rec.fold_tickets;
+    return &foreign_stream_tickets[s];
+  };
+  {
+    std::lock_guard<std::mutex> g(r.mu);
+    if (unsigned *have = *cell_of()) return have;
+  }
+  // first use on this stream: 16 KiB straight from the device (not the pool: the words
+  // live as long as the stream).  When the device is full, the kept by-products go first.
+  void *p = nullptr;
+  if (hipMalloc(&p, kFoldTicketSlots * sizeof(unsigned)) != hipSuccess || !p) {
+    (void)hipGetLastError();
+    p = nullptr;
+    if (drop_all_kept() == 0 || hipMalloc(&p, kFoldTicketSlots * sizeof(unsigned)) != hipSuccess || !p) {
       (void)hipGetLastError();
       return nullptr;
     }
-    hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(kFoldTicketSlots, 256)), dim3(256), 0, s, (unsigned *)p,
-                       kFoldTicketSlots);
-    *cell = (unsigned *)p;
   }
+  hipLaunchKernelGGL(zero_words_kernel, dim3(cdiv(kFoldTicketSlots, 256)), dim3(256), 0, s, (unsigned *)p,
+                     kFoldTicketSlots);
+  std::lock_guard<std::mutex> g(r.mu);
+  unsigned **cell = cell_of();
+  if (*cell) {  // another thread got there first on the same stream
+    (void)hipFree(p);
+    return *cell;
+  }
+  *cell = (unsigned *)p;
   return *cell;
 }
 
@@ -549,16 +560,36 @@ namespace {
 struct Kept {
   const char *lo, *hi;  // bytes of the source array
   void **slot;          // the owner's pointer to the kept block; cleared when the block is dropped
+  size_t block_bytes;   // size of the kept block
+  hipStream_t stream;   // stream whose work produced the block: only a call on it may take it
+  int tag;              // what the block is (the owner's code for form and tile)
 };
 std::mutex kept_mu;
 std::vector<Kept> kept;
 std::atomic<int> kept_count{0};
 std::atomic<long long> kept_total{0}, taken_total{0};  // blocks registered / handed to a later call
+size_t kept_bytes = 0;                                 // with kept_mu held: bytes of all kept blocks
+
+// All kept blocks together may hold at most an eighth of the device's memory (36 GB of
+// 288): the five benchmark configurations keep 1 - 4 GB, so this only bounds a
+// pathological graph (many large Winograd layers whose backward never runs).
+size_t kept_cap() {
+  static const size_t cap = [] {
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) {
+      (void)hipGetLastError();
+      return (size_t)4 << 30;
+    }
+    return total_b / 8;
+  }();
+  return cap;
+}
 
 // with kept_mu held
 void drop_at(size_t i) {
   if (*kept[i].slot) device_free(*kept[i].slot);
   *kept[i].slot = nullptr;
+  kept_bytes -= kept[i].block_bytes;
   kept[i] = kept.back();
   kept.pop_back();
   kept_count.store((int)kept.size(), std::memory_order_release);
@@ -567,7 +598,14 @@ void drop_at(size_t i) {
 
 namespace tf {
 
-void keep_set(void **slot, void *block, const void *src, size_t src_bytes) {
+bool keep_has_room(size_t block_bytes) {
+  const size_t cap = kept_cap();
+  std::lock_guard<std::mutex> g(kept_mu);
+  return kept_bytes + block_bytes <= cap;
+}
+
+void keep_set(void **slot, void *block, size_t block_bytes, const void *src, size_t src_bytes, hipStream_t stream,
+              int tag) {
   std::lock_guard<std::mutex> g(kept_mu);
   for (size_t i = 0; i < kept.size(); ++i)
     if (kept[i].slot == slot) {
@@ -576,16 +614,17 @@ void keep_set(void **slot, void *block, const void *src, size_t src_bytes) {
     }
   *slot = block;
   kept_total.fetch_add(1, std::memory_order_relaxed);
-  kept.push_back({(const char *)src, (const char *)src + src_bytes, slot});
+  kept.push_back({(const char *)src, (const char *)src + src_bytes, slot, block_bytes, stream, tag});
+  kept_bytes += block_bytes;
   kept_count.store((int)kept.size(), std::memory_order_release);
 }
 
-void *keep_take(void **slot, const void *src) {
+void *keep_take(void **slot, const void *src, hipStream_t stream, int tag) {
   if (kept_count.load(std::memory_order_acquire) == 0) return nullptr;
   std::lock_guard<std::mutex> g(kept_mu);
   for (size_t i = 0; i < kept.size(); ++i)
     if (kept[i].slot == slot) {
-      if (kept[i].lo != (const char *)src) return nullptr;
+      if (kept[i].lo != (const char *)src || kept[i].stream != stream || kept[i].tag != tag) return nullptr;
       void *block = *slot;
       *slot = nullptr;
       drop_at(i);
