@@ -30,22 +30,32 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr float kEps = 1e-5f;
+constexpr int kNonTemporal = 2;  // cache-policy operand of a buffer access: a stream that is read once
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- per-activation
 
-// NREG >= N values of one column live in registers.
+// NREG >= N values of one column live in registers.  The three tensors are addressed
+// through buffer descriptors: one per-lane column offset (a VGPR computed once) plus a
+// uniform row offset (a scalar) per access, instead of a 64-bit vector address per
+// access -- the address arithmetic was more than half of the kernel's instructions and
+// cost as many registers as a quarter of the data.  A descriptor covers exactly the N
+// rows, so rows N..NREG-1 read as zero and their stores are dropped by the bounds
+// check: no per-row branch.  Needs NREG * L * 4 < 2^32 (the row offsets are 32-bit).
 // RELU: y = max(bn(x), 0) in the same pass (the fused entry points below).
 template <int NREG, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 float *__restrict__ save_mean,
-                                                                float *__restrict__ save_istd, int N, int64_t L) {
-  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+                                                                float *__restrict__ save_istd, int N, uint32_t L) {
+  const uint32_t l = blockIdx.x * kThreads + threadIdx.x;
   if (l >= L) return;
+  const uint32_t col = l * 4u, row = L * 4u;
+  const __amdgpu_buffer_rsrc_t rx = gemm::make_rsrc(x, (uint32_t)N * row), ry = gemm::make_rsrc(y, (uint32_t)N * row);
   float v[NREG];
 #pragma unroll
-  for (int n = 0; n < NREG; ++n) v[n] = n < N ? __builtin_nontemporal_load(x + (int64_t)n * L + l) : 0.f;
+  for (int n = 0; n < NREG; ++n)
+    v[n] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)col, (int)(n * row), kNonTemporal));
   float s = 0.f;
 #pragma unroll
   for (int n = 0; n < NREG; ++n) s += v[n];
@@ -60,11 +70,11 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   save_mean[l] = mean;
   save_istd[l] = istd;
 #pragma unroll
-  for (int n = 0; n < NREG; ++n)
-    if (n < N) {
-      const float out = (v[n] - mean) * istd;
-      y[(int64_t)n * L + l] = (RELU && out < 0.f) ? 0.f : out;
-    }
+  for (int n = 0; n < NREG; ++n) {
+    const float out = (v[n] - mean) * istd;
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, (RELU && out < 0.f) ? 0.f : out), ry, (int)col,
+                                          (int)(n * row), 0);
+  }
 }
 
 // any N: three sweeps over the column (the second and third hit the cache)
@@ -95,21 +105,25 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_stream_kernel(const fl
 
 // dx = istd/N * (N*dy - sum(dy) - xhat * sum(dy*xhat))
 // RELU: dy is first masked with bn(x) > 0, i.e. the gradient of max(bn(x), 0).
+// Addressing as in the forward kernel; a row beyond N reads dy = 0 and adds nothing.
 template <int NREG, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *__restrict__ x,
                                                                  const float *__restrict__ dy,
                                                                  float *__restrict__ dx,
                                                                  const float *__restrict__ save_mean,
                                                                  const float *__restrict__ save_istd, int N,
-                                                                 int64_t L) {
-  const int64_t l = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+                                                                 uint32_t L) {
+  const uint32_t l = blockIdx.x * kThreads + threadIdx.x;
   if (l >= L) return;
+  const uint32_t col = l * 4u, row = L * 4u, all = (uint32_t)N * row;
+  const __amdgpu_buffer_rsrc_t rx = gemm::make_rsrc(x, all), rg = gemm::make_rsrc(dy, all),
+                               ro = gemm::make_rsrc(dx, all);
   const float mean = save_mean[l], istd = save_istd[l];
   float xh[NREG], g[NREG];
 #pragma unroll
   for (int n = 0; n < NREG; ++n) {
-    xh[n] = n < N ? __builtin_nontemporal_load(x + (int64_t)n * L + l) : mean;
-    g[n] = n < N ? __builtin_nontemporal_load(dy + (int64_t)n * L + l) : 0.f;
+    xh[n] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)col, (int)(n * row), kNonTemporal));
+    g[n] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rg, (int)col, (int)(n * row), kNonTemporal));
   }
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -123,7 +137,8 @@ __global__ __launch_bounds__(kThreads) void bn_pa_backward_kernel(const float *_
   const float scale = istd / m;
 #pragma unroll
   for (int n = 0; n < NREG; ++n)
-    if (n < N) dx[(int64_t)n * L + l] = scale * (m * g[n] - s1 - xh[n] * s2);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, scale * (m * g[n] - s1 - xh[n] * s2)), ro, (int)col,
+                                          (int)(n * row), 0);
 }
 
 template <bool RELU>
@@ -332,6 +347,9 @@ __global__ __launch_bounds__(kThreads) void bn_sp_apply_kernel(const float *__re
   }
 }
 
+// The register kernels address row n at the 32-bit byte offset n * L * 4.
+bool pa_rows_addressable(int nreg, int64_t L) { return (int64_t)nreg * L * 4 < ((int64_t)1 << 32); }
+
 int sp_chunks(int N, int C) {
   // about four workgroups per CU in the partial pass
   int chunks = cdiv((int64_t)num_cus() * 4, C);
@@ -419,12 +437,13 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
     const dim3 grid(cdiv(L, kThreads)), block(kThreads);
     auto run = [&](auto relu_c) {
       constexpr bool RELU = decltype(relu_c)::value;
-      if (d->N <= 32)
-        hipLaunchKernelGGL((bn_pa_forward_kernel<32, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
-      else if (d->N <= 64)
-        hipLaunchKernelGGL((bn_pa_forward_kernel<64, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
-      else if (d->N <= 128)
-        hipLaunchKernelGGL((bn_pa_forward_kernel<128, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, L);
+      const uint32_t l32 = (uint32_t)L;
+      if (d->N <= 32 && pa_rows_addressable(32, L))
+        hipLaunchKernelGGL((bn_pa_forward_kernel<32, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
+      else if (d->N <= 64 && pa_rows_addressable(64, L))
+        hipLaunchKernelGGL((bn_pa_forward_kernel<64, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
+      else if (d->N <= 128 && pa_rows_addressable(128, L))
+        hipLaunchKernelGGL((bn_pa_forward_kernel<128, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
       else
         hipLaunchKernelGGL(bn_pa_forward_stream_kernel<RELU>, grid, block, 0, s, x, y, mean, istd, d->N, L);
     };
@@ -509,12 +528,13 @@ static int bn_backward_impl(const DLArrayHandle input, const DLArrayHandle doutp
       const dim3 grid(cdiv(L, kThreads)), block(kThreads);
       auto run = [&](auto relu_c) {
         constexpr bool RELU = decltype(relu_c)::value;
-        if (d->N <= 32)
-          hipLaunchKernelGGL((bn_pa_backward_kernel<32, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
-        else if (d->N <= 64)
-          hipLaunchKernelGGL((bn_pa_backward_kernel<64, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
-        else if (d->N <= 128)
-          hipLaunchKernelGGL((bn_pa_backward_kernel<128, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
+        const uint32_t l32 = (uint32_t)L;
+        if (d->N <= 32 && pa_rows_addressable(32, L))
+          hipLaunchKernelGGL((bn_pa_backward_kernel<32, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, l32);
+        else if (d->N <= 64 && pa_rows_addressable(64, L))
+          hipLaunchKernelGGL((bn_pa_backward_kernel<64, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, l32);
+        else if (d->N <= 128 && pa_rows_addressable(128, L))
+          hipLaunchKernelGGL((bn_pa_backward_kernel<128, RELU>), grid, block, 0, s, x, dy, dx, mean, istd, d->N, l32);
         else
           hipLaunchKernelGGL(bn_pa_backward_stream_kernel<RELU>, grid, block, 0, s, x, dy, dx, mean, istd, d->N, L);
       };
