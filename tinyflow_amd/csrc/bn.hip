@@ -43,7 +43,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // rows, so rows N..NREG-1 read as zero and their stores are dropped by the bounds
 // check: no per-row branch.  Needs NREG * L * 4 < 2^32 (the row offsets are 32-bit).
 // RELU: y = max(bn(x), 0) in the same pass (the fused entry points below).
-template <int NREG, bool RELU>
+// FULL: N == NREG, no row needs masking in the variance.
+template <int NREG, bool RELU, bool FULL>
 __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 float *__restrict__ save_mean,
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void bn_pa_forward_kernel(const float *__
   float q = 0.f;
 #pragma unroll
   for (int n = 0; n < NREG; ++n) {
-    const float dlt = n < N ? v[n] - mean : 0.f;
+    const float dlt = (FULL || n < N) ? v[n] - mean : 0.f;
     q += dlt * dlt;
   }
   const float istd = 1.0f / sqrtf(q / (float)N + kEps);
@@ -347,6 +348,15 @@ __global__ __launch_bounds__(kThreads) void bn_sp_apply_kernel(const float *__re
   }
 }
 
+template <int NREG, bool RELU>
+void pa_forward(dim3 grid, dim3 block, hipStream_t s, const float *x, float *y, float *mean, float *istd, int N,
+                uint32_t L) {
+  if (N == NREG)
+    hipLaunchKernelGGL((bn_pa_forward_kernel<NREG, RELU, true>), grid, block, 0, s, x, y, mean, istd, N, L);
+  else
+    hipLaunchKernelGGL((bn_pa_forward_kernel<NREG, RELU, false>), grid, block, 0, s, x, y, mean, istd, N, L);
+}
+
 // The register kernels address row n at the 32-bit byte offset n * L * 4.
 bool pa_rows_addressable(int nreg, int64_t L) { return (int64_t)nreg * L * 4 < ((int64_t)1 << 32); }
 
@@ -439,11 +449,11 @@ static int bn_forward_impl(const DLArrayHandle input, DLArrayHandle output, int 
       constexpr bool RELU = decltype(relu_c)::value;
       const uint32_t l32 = (uint32_t)L;
       if (d->N <= 32 && pa_rows_addressable(32, L))
-        hipLaunchKernelGGL((bn_pa_forward_kernel<32, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
+        pa_forward<32, RELU>(grid, block, s, x, y, mean, istd, d->N, l32);
       else if (d->N <= 64 && pa_rows_addressable(64, L))
-        hipLaunchKernelGGL((bn_pa_forward_kernel<64, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
+        pa_forward<64, RELU>(grid, block, s, x, y, mean, istd, d->N, l32);
       else if (d->N <= 128 && pa_rows_addressable(128, L))
-        hipLaunchKernelGGL((bn_pa_forward_kernel<128, RELU>), grid, block, 0, s, x, y, mean, istd, d->N, l32);
+        pa_forward<128, RELU>(grid, block, s, x, y, mean, istd, d->N, l32);
       else
         hipLaunchKernelGGL(bn_pa_forward_stream_kernel<RELU>, grid, block, 0, s, x, y, mean, istd, d->N, L);
     };
