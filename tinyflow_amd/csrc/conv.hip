@@ -31,6 +31,9 @@ using namespace tf;
 using namespace tf::gemm;
 
 namespace {
+typedef float f32x2v __attribute__((ext_vector_type(2)));
+typedef unsigned i32x2v __attribute__((__vector_size__(2 * sizeof(unsigned))));   // operand types of the 8- and 16-byte
+typedef unsigned i32x4v __attribute__((__vector_size__(4 * sizeof(unsigned))));   // buffer builtins
 
 
 // ---- gathered operand, lanes along the pixel index ------------------------------
@@ -508,15 +511,22 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
 // output tile of the same index): the input is a dy, and the launch also writes what
 // grad-filter wants of it, dM[pos][cr][t] = (A y A^T)[pos] with y that inner block --
 // grad-data and grad-filter of one layer then read dy once between them.
+//
+// Addressing: `in`, V and dM are read and written through buffer descriptors, a 32-bit
+// per-lane byte offset plus, for the position planes of V and dM, a uniform plane offset
+// -- one store instruction per value instead of a 64-bit vector address computed for
+// each (every array of a Winograd launch is under 4 GiB: wino_shape bounds the scratch).
 template <int TILE, bool ROW16 = false, bool HALVES = false, bool WITH_DM = false>
 __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ in, float *__restrict__ V, int Cr,
                                                         int H, int W, FastDiv div_tiles, FastDiv div_tw, int pad_h,
-                                                        int pad_w, int T, int Tp, float *__restrict__ dM = nullptr) {
+                                                        int pad_w, int T, int Tp, uint32_t in_bytes,
+                                                        float *__restrict__ dM = nullptr) {
   static_assert(!ROW16 || TILE == 4, "ROW16 is the 6-wide patch whose columns 1..4 start at a multiple of 4");
   constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int cr = blockIdx.y;
   if (t >= (uint32_t)Tp) return;
+  const __amdgpu_buffer_rsrc_t rin = gemm::make_rsrc(in, in_bytes);
   float d[A][A];
 #pragma unroll
   for (int i = 0; i < A; ++i)
@@ -526,7 +536,7 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
     uint32_t img, rem, th, tw;
     div_tiles.divmod(t, img, rem);
     div_tw.divmod(rem, th, tw);
-    const float *plane = in + ((int64_t)img * Cr + cr) * H * W;
+    const uint32_t plane = (img * (uint32_t)Cr + (uint32_t)cr) * (uint32_t)(H * W);  // first element of the plane
     const int h0 = TILE * (int)th - pad_h, w0 = TILE * (int)tw - pad_w;
     if constexpr (ROW16) {
       const int wq = w0 + 1;  // = 4 * tw < W
@@ -534,25 +544,25 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
       for (int i = 0; i < A; ++i) {
         const int h = h0 + i;
         if (h < 0 || h >= H) continue;
-        const float *row = plane + h * W + wq;
-        if (wq > 0) d[i][0] = row[-1];
+        const uint32_t row = (plane + (uint32_t)(h * W + wq)) * 4u;  // byte offset of column wq
+        if (wq > 0) d[i][0] = gemm::buf_load(rin, row - 4u);
         if constexpr (HALVES) {  // the last tile of a row may hold only two columns
-          const float2 lo = *reinterpret_cast<const float2 *>(row);
+          const f32x2v lo = __builtin_bit_cast(f32x2v, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)row, 0, 0));
           d[i][1] = lo.x;
           d[i][2] = lo.y;
           if (wq + 2 < W) {
-            const float2 hi = *reinterpret_cast<const float2 *>(row + 2);
+            const f32x2v hi = __builtin_bit_cast(f32x2v, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)row + 8, 0, 0));
             d[i][3] = hi.x;
             d[i][4] = hi.y;
           }
         } else {
-          const float4 mid = *reinterpret_cast<const float4 *>(row);
+          const gemm::f32x4v mid = gemm::buf_load4(rin, row);
           d[i][1] = mid.x;
           d[i][2] = mid.y;
           d[i][3] = mid.z;
           d[i][4] = mid.w;
         }
-        if (wq + 4 < W) d[i][5] = row[4];
+        if (wq + 4 < W) d[i][5] = gemm::buf_load(rin, row + 16u);
       }
     } else {
 #pragma unroll
@@ -560,7 +570,7 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
 #pragma unroll
         for (int j = 0; j < A; ++j) {
           const int h = h0 + i, x = w0 + j;
-          if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = plane[h * W + x];
+          if (h >= 0 && h < H && x >= 0 && x < W) d[i][j] = gemm::buf_load(rin, (plane + (uint32_t)(h * W + x)) * 4u);
         }
     }
   }
@@ -574,14 +584,17 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
 #pragma unroll
     for (int i = 0; i < A; ++i) r[i][j] = o[i];
   }
-  const int64_t plane_sz = (int64_t)Cr * Tp;
-  float *dst = V + (int64_t)cr * Tp + t;
+  const uint32_t plane_bytes = (uint32_t)Cr * (uint32_t)Tp * 4u;   // one position of V (and of dM)
+  const uint32_t lane_off = ((uint32_t)cr * (uint32_t)Tp + t) * 4u;
+  const __amdgpu_buffer_rsrc_t rv = gemm::make_rsrc(V, (uint32_t)(A * A) * plane_bytes);
 #pragma unroll
   for (int i = 0; i < A; ++i) {
     float o[A];
     Wino<TILE>::bt(r[i], o);
 #pragma unroll
-    for (int j = 0; j < A; ++j) dst[(i * A + j) * plane_sz] = o[j];
+    for (int j = 0; j < A; ++j)
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, o[j]), rv, (int)lane_off,
+                                            (int)((uint32_t)(i * A + j) * plane_bytes), 0);
   }
   if constexpr (WITH_DM) {
     float q[A][TILE];  // A y, column by column
@@ -594,13 +607,15 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
 #pragma unroll
       for (int i = 0; i < A; ++i) q[i][b] = o[i];
     }
-    float *dst2 = dM + (int64_t)cr * Tp + t;
+    const __amdgpu_buffer_rsrc_t rm = gemm::make_rsrc(dM, (uint32_t)(A * A) * plane_bytes);
 #pragma unroll
     for (int i = 0; i < A; ++i) {
       float o[A];
       Wino<TILE>::a(q[i], o);
 #pragma unroll
-      for (int j = 0; j < A; ++j) dst2[(i * A + j) * plane_sz] = o[j];
+      for (int j = 0; j < A; ++j)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, o[j]), rm, (int)lane_off,
+                                              (int)((uint32_t)(i * A + j) * plane_bytes), 0);
     }
   }
 }
@@ -611,18 +626,22 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
 template <int TILE>
 __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, float *__restrict__ out, int Mo,
                                                          int P, int Q, FastDiv div_tiles, FastDiv div_tw, int T,
-                                                         int Tp, bool rows_vec) {
+                                                         int Tp, bool rows_vec, uint32_t out_bytes) {
   constexpr int A = Wino<TILE>::A;
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
   const int mo = blockIdx.y;
   if (t >= (uint32_t)T) return;
-  const int64_t plane_sz = (int64_t)Mo * Tp;
-  const float *src = M + (int64_t)mo * Tp + t;
+  // buffer addressing as in wino_input_kernel: uniform plane offsets for M, uniform row offsets for out
+  const uint32_t plane_bytes = (uint32_t)Mo * (uint32_t)Tp * 4u;
+  const uint32_t lane_off = ((uint32_t)mo * (uint32_t)Tp + t) * 4u;
+  const __amdgpu_buffer_rsrc_t rm = gemm::make_rsrc(M, (uint32_t)(A * A) * plane_bytes);
   float m[A][A];
 #pragma unroll
   for (int i = 0; i < A; ++i)
 #pragma unroll
-    for (int j = 0; j < A; ++j) m[i][j] = __builtin_nontemporal_load(src + (i * A + j) * plane_sz);
+    for (int j = 0; j < A; ++j)
+      m[i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                              rm, (int)lane_off, (int)((uint32_t)(i * A + j) * plane_bytes), 2));
   float s[TILE][A];  // A^T m, column by column
 #pragma unroll
   for (int j = 0; j < A; ++j) {
@@ -637,19 +656,29 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
   div_tiles.divmod(t, img, rem);
   div_tw.divmod(rem, th, tw);
   const int p0 = TILE * (int)th, q0 = TILE * (int)tw;
-  float *dst = out + (((int64_t)img * Mo + mo) * P + p0) * Q + q0;
+  const __amdgpu_buffer_rsrc_t ro = gemm::make_rsrc(out, out_bytes);
+  const uint32_t dst = (((img * (uint32_t)Mo + (uint32_t)mo) * (uint32_t)P + (uint32_t)p0) * (uint32_t)Q + (uint32_t)q0) * 4u;
 #pragma unroll
   for (int a = 0; a < TILE; ++a) {
     if (p0 + a >= P) break;
     float y[TILE];
     Wino<TILE>::at(s[a], y);
+    const int row_off = a * Q * 4;
     if (rows_vec) {
-      if constexpr (TILE == 2) *reinterpret_cast<float2 *>(dst + a * Q) = make_float2(y[0], y[1]);
-      else *reinterpret_cast<float4 *>(dst + a * Q) = make_float4(y[0], y[1], y[2], y[3]);
+      // (the row offset goes into the per-lane offset, not into the scalar operand: 16-byte stores
+      // with a scalar offset register now and then stored a wrong first word at full-size layers,
+      // when the next row's arithmetic reused the data registers)
+      if constexpr (TILE == 2) {
+        const f32x2v v = {y[0], y[1]};
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(i32x2v, v), ro, (int)dst + row_off, 0, 0);
+      } else {
+        const gemm::f32x4v v = {y[0], y[1], y[2], y[3]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4v, v), ro, (int)dst + row_off, 0, 0);
+      }
     } else {
 #pragma unroll
       for (int b2 = 0; b2 < TILE; ++b2)
-        if (q0 + b2 < Q) dst[a * Q + b2] = y[b2];
+        if (q0 + b2 < Q) gemm::buf_store(ro, dst + (uint32_t)(row_off + b2 * 4), y[b2]);
     }
   }
 }
@@ -709,14 +738,17 @@ __global__ __launch_bounds__(256) void wino_dy_kernel(const float *__restrict__ 
 #pragma unroll
     for (int i = 0; i < A; ++i) r[i][b] = o[i];
   }
-  const int64_t plane_sz = (int64_t)K * Tp;
-  float *dst = dM + (int64_t)k * Tp + t;
+  const uint32_t plane_bytes = (uint32_t)K * (uint32_t)Tp * 4u;
+  const uint32_t lane_off = ((uint32_t)k * (uint32_t)Tp + t) * 4u;
+  const __amdgpu_buffer_rsrc_t rm = gemm::make_rsrc(dM, (uint32_t)(A * A) * plane_bytes);
 #pragma unroll
   for (int i = 0; i < A; ++i) {
     float o[A];
     Wino<TILE>::a(r[i], o);
 #pragma unroll
-    for (int j = 0; j < A; ++j) dst[(i * A + j) * plane_sz] = o[j];
+    for (int j = 0; j < A; ++j)
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, o[j]), rm, (int)lane_off,
+                                            (int)((uint32_t)(i * A + j) * plane_bytes), 0);
   }
 }
 
@@ -1193,18 +1225,19 @@ ConvPlan plan_wgrad(const ConvDesc *d) {
 // Nothing is kept under a device-memory budget or with TINYFLOW_KEEP_TRANSFORMED_INPUT=0.
 // Launches the input transform x -> V (and, with dM, the grad-filter form of the same
 // array, see WITH_DM) in the variant the row length and alignment allow.
-void launch_wino_input(int tile, const float *in, float *V, float *dM, int Cr, int H, int W, int pad_h, int pad_w,
-                       const FastDiv &div_tiles, const FastDiv &div_tw, int T, int Tp, hipStream_t s) {
+void launch_wino_input(int tile, const float *in, float *V, float *dM, int images, int Cr, int H, int W, int pad_h,
+                       int pad_w, const FastDiv &div_tiles, const FastDiv &div_tw, int T, int Tp, hipStream_t s) {
   const dim3 grid(cdiv(Tp, 256), Cr), block(256);
+  const uint32_t in_bytes = (uint32_t)((size_t)images * Cr * H * W * sizeof(float));  // under 4 GiB: smaller than V
   if (tile == 2) {
     hipLaunchKernelGGL(wino_input_kernel<2>, grid, block, 0, s, in, V, Cr, H, W, div_tiles, div_tw, pad_h, pad_w, T, Tp,
-                       nullptr);
+                       in_bytes, nullptr);
     return;
   }
   const bool row16 = pad_w == 1 && W % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
   const bool halves = !row16 && pad_w == 1 && W % 2 == 0 && (reinterpret_cast<uintptr_t>(in) & 7u) == 0;
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, block, 0, s, in, V, Cr, H, W, div_tiles, div_tw, pad_h, pad_w, T, Tp, dM);
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, in, V, Cr, H, W, div_tiles, div_tw, pad_h, pad_w, T, Tp, in_bytes, dM);
   };
   if (dM) {
     if (row16) go(wino_input_kernel<4, true, false, true>);
@@ -1279,7 +1312,7 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
       hipLaunchKernelGGL(wino_filter_kernel<4>, fgrid, block, 0, s, filter, U, d->K, d->C, dgrad, U_for_dgrad);
   }
   if (!V_kept)
-    launch_wino_input(w.tile, in, V, dM_for_wgrad, w.Cr, w.in_h, w.in_w, w.pad_h, w.pad_w, div_tiles, div_tw, w.T, w.Tp,
+    launch_wino_input(w.tile, in, V, dM_for_wgrad, d->N, w.Cr, w.in_h, w.in_w, w.pad_h, w.pad_w, div_tiles, div_tw, w.T, w.Tp,
                       s);
   with_tile(plan.bm, plan.bn, [&](auto bm_c, auto bn_c, auto bk_c) {
     constexpr int BM = decltype(bm_c)::value, BN = decltype(bn_c)::value, BK = decltype(bk_c)::value;
@@ -1297,12 +1330,13 @@ int run_winograd(ConvDesc *d, bool dgrad, const ConvPlan &plan, const float *in,
     }
   }, run_depth(plan.bm, plan.bn, w.Cr));
   const bool rows_vec = w.out_w % w.tile == 0 && (reinterpret_cast<uintptr_t>(out) & (uintptr_t)(4 * w.tile - 1)) == 0;
+  const uint32_t out_bytes = (uint32_t)((size_t)d->N * w.Mo * w.out_h * w.out_w * sizeof(float));  // smaller than M
   if (w.tile == 2)
     hipLaunchKernelGGL(wino_output_kernel<2>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
-                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
+                       div_tiles, div_tw, w.T, w.Tp, rows_vec, out_bytes);
   else
     hipLaunchKernelGGL(wino_output_kernel<4>, ogrid, block, 0, s, (const float *)Mt, out, w.Mo, w.out_h, w.out_w,
-                       div_tiles, div_tw, w.T, w.Tp, rows_vec);
+                       div_tiles, div_tw, w.T, w.Tp, rows_vec, out_bytes);
   device_free(scratch);
   if (U_kept) device_free(U_kept);
   if (V_kept) device_free(V_kept);
@@ -1356,11 +1390,11 @@ int run_winograd_wgrad(ConvDesc *d, const ConvPlan &plan, const float *x, const 
   const bool rows_vec = d->Q % w.tile == 0 && (reinterpret_cast<uintptr_t>(dy) & (uintptr_t)(4 * w.tile - 1)) == 0;
   const dim3 block(256);
   if (!kept_V)
-    launch_wino_input(w.tile, x, V, nullptr, d->C, d->H, d->W, d->pad_h, d->pad_w, div_tiles, div_tw, w.T, w.Tp, s);
+    launch_wino_input(w.tile, x, V, nullptr, d->N, d->C, d->H, d->W, d->pad_h, d->pad_w, div_tiles, div_tw, w.T, w.Tp, s);
   if (dM_kept)
     ;  // dM is grad-data's by-product
   else if (V_for_dgrad)  // one pass over dy writes grad-data's V (kept) and dM
-    launch_wino_input(4, dy, V_for_dgrad, dM, d->K, d->P, d->Q, 2 - d->pad_h, 2 - d->pad_w, div_tiles, div_tw, w.T, w.Tp,
+    launch_wino_input(4, dy, V_for_dgrad, dM, d->N, d->K, d->P, d->Q, 2 - d->pad_h, 2 - d->pad_w, div_tiles, div_tw, w.T, w.Tp,
                       s);
   else if (w.tile == 2)
     hipLaunchKernelGGL(wino_dy_kernel<2>, dim3(cdiv(w.Tp, 256), d->K), block, 0, s, dy, dM, d->K, d->P, d->Q, div_tiles,
