@@ -74,7 +74,9 @@ def stream_handle(stream_cell):
     return ctypes.cast(stream_cell, ctypes.POINTER(ctypes.c_void_p))[0]
 
 
-TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "resnet50_b64_train_step_hbm_traffic.txt")
+def traffic_summary_path(config, batch):
+    """The committed counter summary of one workload (written from two rocprofv3 --pmc runs of this script)."""
+    return os.path.join(ROOT, "profiles", "%s_b%d_train_step_hbm_traffic.txt" % (config, batch))
 
 
 def _normalise_symbol(name):
@@ -82,15 +84,16 @@ def _normalise_symbol(name):
     return name.replace(" >", ">").replace(", ", ",").strip()
 
 
-def measured_traffic_bytes():
+def measured_traffic_bytes(config, batch):
     """{kernel symbol: HBM bytes per launch (reads + writes)} from the committed summary of
     the two rocprofv3 counter runs of this script (FETCH_SIZE, WRITE_SIZE, each scaled by
     what the same counter reads for a copy of known size; the summary states the commands
-    and the factors).  It covers --config resnet50 --batch 64 in per-activation mode; a
-    symbol the summary does not list (a kernel changed since the counter run) reads null."""
+    and the factors).  One summary per workload (configuration at its own batch size, per-
+    activation batch norm); a workload without one, or a symbol its summary does not list
+    (a kernel changed since the counter run), reads null."""
     table = {}
     try:
-        with open(TRAFFIC_SUMMARY) as fh:
+        with open(traffic_summary_path(config, batch)) as fh:
             lines = fh.read().splitlines()
     except OSError:
         return table
@@ -491,9 +494,19 @@ def main():
 
     stats = timer.collect(pair_overhead)
     gpu_step_ms = gpu_ms / args.steps
-    default_workload = ((args.config, args.batch, args.bn_mode) == ("resnet50", 64, "pre_activation")
-                        and not args.mem_limit_gb)
-    traffic = measured_traffic_bytes() if default_workload else {}
+    traffic = measured_traffic_bytes(args.config, args.batch) if args.bn_mode == "pre_activation" else {}
+    RIDGE = MFMA_FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBPS * 1e9)   # flop per HBM byte where the two roofs meet
+
+    def bound_of(name, launches, total_ms, total_flops):
+        """Which roof bounds a contraction symbol: with its counter traffic known, a launch that executes fewer
+        flops per HBM byte than the ridge (19.7) is priced against HBM, not against the matrix pipes."""
+        nbytes = traffic.get(_normalise_symbol(name))
+        if not nbytes:
+            return {"bound": "mfma", "traffic": None}
+        intensity = total_flops / launches / nbytes
+        gbps = nbytes * launches / (total_ms * 1e-3) / 1e9
+        return {"bound": "hbm" if intensity < RIDGE else "mfma", "traffic": nbytes, "flop_per_hbm_byte": intensity,
+                "hbm_GBps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
 
     def symbol_roofline(which, name, launches, total_ms, total_flops):
         achieved = total_flops / (total_ms * 1e-3) / 1e12
@@ -501,6 +514,7 @@ def main():
             "bound": "mfma", "pass": PASS_NAMES[which], "kernel": name, "achieved": achieved,
             "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
             "traffic": traffic.get(_normalise_symbol(name)),
+            "against_hbm": bound_of(name, launches, total_ms, total_flops),
             "flops_per_launch": total_flops / launches,
             "launches": launches, "avg_launch_ms": total_ms / launches,
             "share_of_step": total_ms / event_steps / gpu_step_ms, "steps_with_events": event_steps,
@@ -527,9 +541,10 @@ def main():
             "executed_tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
             "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "ms_per_step": ms / event_steps,
             "launches_per_step": sum(v[0] for _, v in rows) / event_steps, "symbols": len(rows),
-            "slowest_symbol": {"kernel": slow_name, "tflops": slow[2] / (slow[1] * 1e-3) / 1e12,
-                               "frac": slow[2] / (slow[1] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
-                               "ms_per_step": slow[1] / event_steps, "launches_per_step": slow[0] / event_steps},
+            "slowest_symbol": dict({"kernel": slow_name, "tflops": slow[2] / (slow[1] * 1e-3) / 1e12,
+                                    "frac": slow[2] / (slow[1] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
+                                    "ms_per_step": slow[1] / event_steps, "launches_per_step": slow[0] / event_steps},
+                                   **bound_of(slow_name, slow[0], slow[1], slow[2])),
         }
 
     # `roofline`: the backward contraction kernel (grad-data or grad-filter) with the most
@@ -560,7 +575,9 @@ def main():
                                  % (PASS_NAMES[which], k, n / event_steps, ms / event_steps, fl / (ms * 1e-3) / 1e12))
 
     result = {
-        "metric": "train imgs/sec ResNet-50 b64 fp32 fwd+bwd; bwd kernel % of HBM/MFMA peak",
+        "metric": ("train imgs/sec ResNet-50 b64 fp32 fwd+bwd; bwd kernel % of HBM/MFMA peak"
+                   if (args.config, args.batch) == ("resnet50", 64)
+                   else "train imgs/sec %s b%d fp32 fwd+bwd; bwd kernel %% of HBM/MFMA peak" % (args.config, args.batch)),
         "value": imgs_per_sec, "unit": "imgs/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",

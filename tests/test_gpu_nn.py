@@ -271,6 +271,55 @@ def test_batch_norm_with_mean_far_from_zero(rt, mode):
     parity.compare(gdx.asnumpy(), dx_ref, dx32, "batch norm backward, %s, |mean| >> std" % mode, "bn bwd offset", K_BN)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [5, 33, 65, 100])
+def test_batch_norm_with_fewer_rows_than_its_registers_writes_only_its_rows(rt, rows):
+    """The per-activation kernels hold 32, 64 or 128 rows and leave the rows a batch does not
+    have to the bounds check of their buffer descriptors.  The arrays handed over here are the
+    first `rows` rows of larger allocations filled with a sentinel: after forward and backward
+    the rows behind the batch must still hold it (a store that escaped the check would land
+    exactly there), and the batch's own rows must equal a run on arrays of their own."""
+    import ctypes
+    from tinyflow_amd import gpu_op, ndarray
+    L, slack, sentinel = 3 * 5 * 7, 128, -7.5
+    rng = np.random.RandomState(24)
+    x = rng.normal(0, 1, (rows, 3, 5, 7)).astype(np.float32)
+    dy = rng.normal(0, 1, (rows, 3, 5, 7)).astype(np.float32)
+
+    def view(big, values=None):
+        """NDArray over the first `rows` rows of `big` (not an owner: never freed through the library)."""
+        if values is not None:
+            host = np.full((rows + slack, L), sentinel, np.float32)
+            host[:rows] = values.reshape(rows, L)
+            big._sync_copyfrom(host)
+        shape = (ctypes.c_int64 * 4)(rows, 3, 5, 7)
+        arr = ndarray.DLArray(big.handle.contents.data, rt.ctx, 4, shape)
+        v = ndarray.NDArray(ctypes.pointer(arr))
+        v.is_freed = True            # the storage belongs to `big`
+        return v, (arr, shape)
+
+    bigs = [ndarray.empty((rows + slack, L), rt.ctx) for _ in range(4)]
+    (vx, k0), (vdy, k1) = view(bigs[0], x), view(bigs[1], dy)
+    (vy, k2), (vdx, k3) = view(bigs[2], np.zeros_like(x)), view(bigs[3], np.zeros_like(x))
+    mp, vp, lst = gpu_op.bn_get_cudnnlist(x.shape, "NCHW", "pre_activation")
+    assert gpu_op.bn_forward(vx, vy, "pre_activation", 0, mp, vp, lst, rt.cudnn, rt.stream) == 0
+    assert gpu_op.bn_backward(vx, vdy, vdx, "pre_activation", mp, vp, lst, rt.cudnn, rt.stream) == 0
+    got_y, got_dx = bigs[2].asnumpy(), bigs[3].asnumpy()
+    assert np.all(got_y[rows:] == sentinel) and np.all(got_dx[rows:] == sentinel)
+    assert np.all(bigs[0].asnumpy()[rows:] == sentinel) and np.all(bigs[1].asnumpy()[rows:] == sentinel)
+    # the same call on arrays of their own
+    gx, gdy = _gpu(x, rt), _gpu(dy, rt)
+    gy, gdx = ndarray.empty(x.shape, rt.ctx), ndarray.empty(x.shape, rt.ctx)
+    mp2, vp2, lst2 = gpu_op.bn_get_cudnnlist(x.shape, "NCHW", "pre_activation")
+    gpu_op.bn_forward(gx, gy, "pre_activation", 0, mp2, vp2, lst2, rt.cudnn, rt.stream)
+    gpu_op.bn_backward(gx, gdy, gdx, "pre_activation", mp2, vp2, lst2, rt.cudnn, rt.stream)
+    assert got_y[:rows].tobytes() == gy.asnumpy().tobytes()
+    assert got_dx[:rows].tobytes() == gdx.asnumpy().tobytes()
+    y_ref = O.batch_norm_forward(x.astype(np.float64), "pre_activation")[0]
+    np.testing.assert_allclose(got_y[:rows].reshape(x.shape), y_ref, rtol=1e-3, atol=2e-5)
+    del k0, k1, k2, k3
+
+
 # ------------------------------------------------------- dropout, concatenation
 
 @pytest.mark.gpu
