@@ -361,7 +361,7 @@ def main():
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="do not record per-convolution HIP events in the timed region")
     ap.add_argument("--breakdown", action="store_true", help="print per-variant conv times to stderr")
-    ap.add_argument("--event-every", type=int, default=4,
+    ap.add_argument("--event-every", type=int, default=10,
                     help="record the per-kernel HIP events in every n-th timed step only (each event pair "
                          "costs a few microseconds of queue time, which would otherwise weigh on `value`)")
     ap.add_argument("--copy-calibration", action="store_true",
