@@ -223,14 +223,17 @@ class HbmTimer(object):
         self.enabled = False
         self.pairs = []
         self.streamless = None   # stream the library uses for entry points without a stream argument
+        self.mask_counts = gpu_op.relu_mask_counts
         n = lambda a: int(np.prod(a.shape))
         bn_b = (8, 12) if bn_mode == "pre_activation" else (12, 20)
         table = {
             # op: bytes moved by one call, from its array arguments
             "bn_forward": lambda a: bn_b[0] * n(a[0]),
             "bn_backward": lambda a: bn_b[1] * n(a[0]),
-            "activation_forward": lambda a: 8 * n(a[0]),
-            "activation_backward": lambda a: 12 * n(a[0]),
+            # a ReLU forward call that keeps its sign bits writes one more bit per element, and the
+            # backward call that uses them reads dy and the bits instead of dy and x
+            "activation_forward": lambda a, bits=False: (8.125 if bits else 8) * n(a[0]),
+            "activation_backward": lambda a, bits=False: (8.125 if bits else 12) * n(a[0]),
             "matrix_elementwise_add": lambda a: 12 * n(a[2]),
             "pooling_2d_backward": lambda a: 4 * (n(a[0]) + n(a[1]) + n(a[2]) + n(a[3])),
             "sgd_update": lambda a: 12 * n(a[0]),
@@ -247,10 +250,12 @@ class HbmTimer(object):
             s = self.streamless if name == "sgd_compute_o" else stream_handle(args[-1])
             e0 = self.pool.pop() if self.pool else self.hip.event()
             e1 = self.pool.pop() if self.pool else self.hip.event()
+            counts = self.mask_counts() if name.startswith("activation_") else None
             self.hip.record(e0, s)
             ret = fn(*args)
             self.hip.record(e1, s)
-            self.pairs.append((name, nbytes(args), e0, e1))
+            moved = nbytes(args) if counts is None else nbytes(args, self.mask_counts() != counts)
+            self.pairs.append((name, moved, e0, e1))
             return ret
         return timed
 

@@ -308,6 +308,17 @@ int DLGpuActivationBackward(const DLArrayHandle input, DLArrayHandle dinput,
                             const DLArrayHandle output, const DLArrayHandle doutput,
                             int activationMode, void ***list, void **handle, void **stream);
 
+/* No counterpart in the reference: introspection for tests and for the benchmark's
+ * byte accounting.  Once a ReLU descriptor has seen a backward call, its forward calls
+ * also write one bit per element (x > 0) into a block of the library's own, and the
+ * backward call of the same step on the same, unmodified x reads dy and the bits
+ * instead of dy and x, with the same result bit for bit (any entry point that writes
+ * or frees x drops the bits, and the call reads x as before).  Nothing is kept under a
+ * device-memory budget or with TINYFLOW_KEEP_RELU_MASK=0 in the environment.
+ * Reports how many forward calls kept their bits and how many backward calls used
+ * them since the library was loaded; either pointer may be NULL. */
+int DLGpuReluMaskCounts(long long *kept, long long *used);
+
 /* ------------------------------------------------------ batch normalisation */
 
 /* gamma = 1, beta = 0, eps = 1e-5, biased variance; no running statistics.

@@ -450,6 +450,120 @@ def test_relu_masks_at_full_activation_size(rt):
     assert gy.asnumpy().tobytes() == want_y.tobytes() and gdx.asnumpy().tobytes() == want_dx.tobytes()
 
 
+def _relu_mask_counts():
+    from tinyflow_amd import gpu_op
+    return gpu_op.relu_mask_counts()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(8, 64, 56, 56), (3, 7, 60, 56), (1, 1, 256, 257), (64, 256, 56, 56)], ids=str)
+def test_relu_backward_from_kept_sign_bits_is_bit_identical(rt, shape):
+    """From a descriptor's second step on, the ReLU forward call keeps one bit per element
+    and the backward call reads dy and the bits instead of dy and x.  Same bytes as the
+    oracle and as the first step (which read x), also with exact zeros, negative zeros,
+    a ragged last workgroup, and different data in each step."""
+    from tinyflow_amd import gpu_op, ndarray
+    gen = np.random.default_rng(17)
+    lst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
+    gy, gdx = ndarray.empty(shape, rt.ctx), ndarray.empty(shape, rt.ctx)
+    for step in range(3):
+        x = gen.standard_normal(shape, dtype=np.float32)
+        x.reshape(-1)[::7] = 0.0
+        x.reshape(-1)[3::11] = -0.0
+        dy = gen.standard_normal(shape, dtype=np.float32)
+        gx, gdy = ndarray.array(x, rt.ctx), ndarray.array(dy, rt.ctx)
+        gpu_op.array_set(gy, np.nan, rt.stream)
+        gpu_op.array_set(gdx, np.nan, rt.stream)
+        kept0, used0 = _relu_mask_counts()
+        gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+        gpu_op.activation_backward(gx, gdx, gy, gdy, "relu", lst, rt.cudnn, rt.stream)
+        kept1, used1 = _relu_mask_counts()
+        assert (kept1 - kept0, used1 - used0) == ((0, 0) if step == 0 else (1, 1)), step
+        assert gy.asnumpy().tobytes() == O.relu(x).tobytes(), step
+        assert gdx.asnumpy().tobytes() == O.relu_gradient(x, dy).tobytes(), step
+
+
+@pytest.mark.gpu
+def test_kept_relu_sign_bits_follow_the_input_array(rt):
+    """The kept bits describe x as the forward call read it.  A backward call must not use
+    them once x was overwritten, when it is given another array, under a device-memory
+    budget, for an array too small or of a length that is no multiple of four, or when
+    the forward call ran in place; each time it reads x and gives the oracle's bytes."""
+    from tinyflow_amd import gpu_op, ndarray
+    gen = np.random.default_rng(19)
+    shape = (4, 32, 28, 28)
+
+    def fresh(shape):
+        x = gen.standard_normal(shape, dtype=np.float32)
+        dy = gen.standard_normal(shape, dtype=np.float32)
+        return x, dy, ndarray.array(x, rt.ctx), ndarray.array(dy, rt.ctx)
+
+    def backward(lst, gx, gy, gdy, shape):
+        gdx = ndarray.empty(shape, rt.ctx)
+        gpu_op.array_set(gdx, np.nan, rt.stream)
+        gpu_op.activation_backward(gx, gdx, gy, gdy, "relu", lst, rt.cudnn, rt.stream)
+        return gdx.asnumpy()
+
+    lst = gpu_op.activation_get_cudnnlist(shape, "NCHW", "relu")
+    gy = ndarray.empty(shape, rt.ctx)
+    x, dy, gx, gdy = fresh(shape)
+    gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+    assert backward(lst, gx, gy, gdy, shape).tobytes() == O.relu_gradient(x, dy).tobytes()   # the descriptor has now seen a backward call
+
+    # x overwritten between the two calls
+    kept0, used0 = _relu_mask_counts()
+    gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+    x2 = -x
+    gx[:] = x2
+    assert backward(lst, gx, gy, gdy, shape).tobytes() == O.relu_gradient(x2, dy).tobytes()
+    assert _relu_mask_counts() == (kept0 + 1, used0)
+
+    # another array of the same shape given to the backward call
+    gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+    x3, _, gx3, _ = fresh(shape)
+    assert backward(lst, gx3, gy, gdy, shape).tobytes() == O.relu_gradient(x3, dy).tobytes()
+    assert _relu_mask_counts() == (kept0 + 2, used0)
+    # the bits stay with the array they describe, untouched since: its own backward call uses them
+    assert backward(lst, gx, gy, gdy, shape).tobytes() == O.relu_gradient(x2, dy).tobytes()
+    assert _relu_mask_counts() == (kept0 + 2, used0 + 1)
+
+    # the bits of an array whose storage was released and handed out again are gone
+    gpu_op.activation_forward(gx, gy, "relu", lst, rt.cudnn, rt.stream)
+    del gx
+    x4, _, gx4, _ = fresh(shape)
+    assert backward(lst, gx4, gy, gdy, shape).tobytes() == O.relu_gradient(x4, dy).tobytes()
+    assert _relu_mask_counts() == (kept0 + 3, used0 + 1)
+
+    # under a device-memory budget nothing is kept
+    kept0, used0 = _relu_mask_counts()
+    in_use = gpu_op.device_memory_stats()[1]
+    gpu_op.set_device_memory_limit(in_use + (1 << 30))
+    try:
+        gpu_op.activation_forward(gx4, gy, "relu", lst, rt.cudnn, rt.stream)
+        assert backward(lst, gx4, gy, gdy, shape).tobytes() == O.relu_gradient(x4, dy).tobytes()
+    finally:
+        gpu_op.set_device_memory_limit(0)
+    assert _relu_mask_counts() == (kept0, used0)
+
+    # small arrays and lengths that are no multiple of four take the plain kernels
+    for small in [(2, 3, 5, 5), (1, 1, 257, 257)]:
+        slst = gpu_op.activation_get_cudnnlist(small, "NCHW", "relu")
+        sy = ndarray.empty(small, rt.ctx)
+        for _ in range(2):
+            xs, dys, gxs, gdys = fresh(small)
+            gpu_op.activation_forward(gxs, sy, "relu", slst, rt.cudnn, rt.stream)
+            assert sy.asnumpy().tobytes() == O.relu(xs).tobytes()
+            assert backward(slst, gxs, sy, gdys, small).tobytes() == O.relu_gradient(xs, dys).tobytes()
+    assert _relu_mask_counts() == (kept0, used0)
+
+    # in place: y overwrites x, and the backward call is then given y, whose sign is x's
+    x5, dy5, gx5, gdy5 = fresh(shape)
+    gpu_op.activation_forward(gx5, gx5, "relu", lst, rt.cudnn, rt.stream)
+    assert gx5.asnumpy().tobytes() == O.relu(x5).tobytes()
+    assert backward(lst, gx5, gx5, gdy5, shape).tobytes() == O.relu_gradient(x5, dy5).tobytes()
+    assert _relu_mask_counts() == (kept0, used0)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(64, 64, 28, 28), (5, 3, 4, 4), (128, 8, 6, 6), (200, 4, 3, 3), (64, 256, 56, 56)],
                          ids=str)

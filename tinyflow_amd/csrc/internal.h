@@ -151,6 +151,11 @@ struct ActDesc {
   int magic;
   int mode;
   int64_t n, inner;    // n instances of `inner` = c*h*w elements
+  // ReLU only: one bit per element, x > 0, written by the forward call beside y and
+  // kept for the backward call of the same step, which then reads dy and the bits
+  // (8.125 bytes per element) instead of dy and x (12).  Owned by keep_set / keep_take.
+  void *kept_mask = nullptr;
+  bool backward_seen = false;   // a forward call keeps bits only once a backward call has used this descriptor
 };
 
 struct BNDesc {

@@ -524,6 +524,14 @@ def set_device_memory_limit(nbytes):
     check_call(_LIB.DLGpuSetDeviceMemoryLimit(ctypes.c_int64(int(nbytes or 0))))
 
 
+def relu_mask_counts():
+    """(kept, used): ReLU forward calls that kept their sign bits for the backward call, and
+    backward calls that read those bits instead of x, since the library was loaded."""
+    kept, used = ctypes.c_longlong(0), ctypes.c_longlong(0)
+    check_call(_LIB.DLGpuReluMaskCounts(ctypes.byref(kept), ctypes.byref(used)))
+    return kept.value, used.value
+
+
 def device_memory_stats(reset_peak=False):
     """(reserved, in_use, peak_in_use) bytes of the device allocator."""
     vals = [ctypes.c_int64(0) for _ in range(3)]
